@@ -1,0 +1,125 @@
+/*
+ * fa2.h - C ABI of libfa2_hip.so: Flash-Attention-2 forward and backward for
+ * AMD MI355X (gfx950), hand-written HIP kernels.
+ *
+ * This is the operator boundary of the hot path.  It takes the place of the
+ * XLA custom calls that the reference emits through
+ * eformer.callib.triton_call(...) at
+ *   jax_flash_attn2/flash_attention_triton/_forward_triton.py:547-588   (forward)
+ *   jax_flash_attn2/flash_attention_triton/_backward_triton.py:1049-1080 (delta pre-pass)
+ *   jax_flash_attn2/flash_attention_triton/_backward_triton.py:1082-1154 (dK/dV/dQ)
+ * Arrays become device pointers, Python scalars become struct fields, outputs
+ * are caller-allocated buffers.  The library never allocates, frees or
+ * synchronises; every launch goes to the caller's stream.
+ *
+ * Tensor layout (same as the reference API, flash_attention.py:186-187):
+ *   q, o, dO, dq : [B, Sq, Hq,  D]     k, v, dk, dv : [B, Sk, Hkv, D]
+ * with arbitrary element strides for batch / sequence / head and a unit
+ * stride on D (the reference assumes the same, _forward_triton.py:296,304,312).
+ * q-head h reads kv-head h / (Hq / Hkv)  (_forward_triton.py:263-264).
+ */
+#ifndef FA2_H_
+#define FA2_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Element types; the values mirror dtype_index() in
+ * jax_flash_attn2/flash_attention_triton/_utils.py:75-82. */
+enum { FA2_FP16 = 1, FA2_BF16 = 2, FA2_FP32 = 3 /* bias only */ };
+
+/* Return codes. 0 = success, negative = error; nothing is launched on error. */
+enum {
+	FA2_OK = 0,
+	FA2_EINVAL_STRUCT = -1,   /* NULL params or struct_size too small            */
+	FA2_EINVAL_DTYPE = -2,    /* q/k/v dtype not fp16/bf16 (_forward_triton.py:494-495) */
+	FA2_EINVAL_SHAPE = -3,    /* non-positive dimension                          */
+	FA2_EINVAL_HEADS = -4,    /* Hq % Hkv != 0 (flash_attention.py:189-193)      */
+	FA2_EINVAL_PTR = -5,      /* required pointer is NULL or not 16-byte aligned */
+	FA2_EINVAL_STRIDE = -6,   /* stride not a multiple of 8 elements             */
+	FA2_EINVAL_DROPOUT = -7,  /* p_drop outside [0, 1)                           */
+	FA2_EINVAL_BIAS = -8,     /* bias dtype / stride invalid                     */
+	FA2_EINVAL_MASK = -9,     /* seqlens given together with bias or with Sq != Sk
+	                             (_forward_triton.py:474-481)                    */
+	FA2_EUNSUPPORTED = -10,   /* head dim not in {64, 128, 256}                  */
+	FA2_ESCRATCH = -11,       /* backward scratch missing or too small           */
+	FA2_EHIP = -12            /* HIP runtime reported a launch error             */
+};
+
+typedef struct fa2_tensor {
+	void* ptr;          /* device pointer, 16-byte aligned                */
+	int64_t stride_b;   /* element stride between batches                 */
+	int64_t stride_s;   /* element stride between sequence positions      */
+	int64_t stride_h;   /* element stride between heads; D stride is 1    */
+} fa2_tensor;
+
+typedef struct fa2_params {
+	uint32_t struct_size;   /* = sizeof(fa2_params), checked first        */
+	int32_t dtype;          /* FA2_FP16 | FA2_BF16 for q,k,v,o,dO,dq,dk,dv */
+	int32_t B, Sq, Sk, Hq, Hkv, D;
+	int32_t causal;         /* bottom-right aligned: j <= i + Sk - Sq
+	                           (_forward_triton.py:127-132)                */
+	float scale;            /* softmax scale, applied to q.k^T             */
+	float p_drop;           /* dropout probability in [0,1)                */
+	uint64_t seed;          /* Philox key for the dropout keep-mask        */
+
+	fa2_tensor q, k, v, o;  /* o is written by fa2_fwd, read by fa2_bwd    */
+	float* lse;             /* [B, Hq, Sq] fp32, natural-log logsumexp; -inf for
+	                           rows without any allowed key.  Written by fa2_fwd,
+	                           read by fa2_bwd.                            */
+
+	/* Optional additive bias [B|1, Hq|Hkv|1, Sq, Sk], unit stride on Sk.
+	 * stride 0 on batch / head = broadcast (calc_bias_strides, _utils.py:151-193).
+	 * bias_group != 0: the head axis has Hkv entries and q-head h reads entry
+	 * h / (Hq/Hkv) (flash_attention.py:161-164 materialises this repeat).   */
+	const void* bias;       /* NULL = no bias                              */
+	int32_t bias_dtype;     /* FA2_FP16 | FA2_BF16 | FA2_FP32              */
+	int32_t bias_group;
+	int64_t bias_stride_b, bias_stride_h, bias_stride_m;
+
+	/* Optional per-batch valid length (the reference's 2-D right-padded
+	 * attention_mask reduced to lengths, _forward_triton.py:499-510): keys
+	 * j >= seqlens[b] are masked, query rows i >= seqlens[b] give zeros.
+	 * Requires Sq == Sk and no bias.                                       */
+	const int32_t* seqlens; /* [B] int32 on device, NULL = all full        */
+
+	/* Backward only. */
+	fa2_tensor dout;        /* dO, read                                    */
+	fa2_tensor dq, dk, dv;  /* written; dk/dv already summed over each KV group */
+	void* scratch;          /* >= fa2_bwd_scratch_bytes(p) bytes, 256-byte aligned */
+	uint64_t scratch_bytes;
+} fa2_params;
+
+/* O = softmax(scale q k^T + bias, masked) v, with dropout; writes o and lse.
+ * Replaces the `_attn_fwd` custom call (_forward_triton.py:547-588). */
+int fa2_fwd(const fa2_params* p, void* hip_stream);
+
+/* dq, dk, dv from (q, k, v, o, lse, dO).  Replaces the `_attn_bwd_preprocess`
+ * and `_attn_bwd` custom calls and the XLA reduce over the KV group
+ * (_backward_triton.py:1049-1161). */
+int fa2_bwd(const fa2_params* p, void* hip_stream);
+
+/* Bytes of scratch fa2_bwd needs for these dimensions (0 on invalid params). */
+size_t fa2_bwd_scratch_bytes(const fa2_params* p);
+
+/* keep[b,h,i,j] (uint8, contiguous [B,Hq,Sq,Sk]) of the dropout mask the
+ * kernels apply for (seed, p_drop); for validation against the Philox
+ * definition.  Counterpart of `tl.rand(seed, offs) > p`
+ * (_forward_triton.py:140-143). Uses B, Hq, Sq, Sk, p_drop, seed only. */
+int fa2_dropout_mask(const fa2_params* p, uint8_t* keep, void* hip_stream);
+
+/* Validate params exactly as fa2_fwd / fa2_bwd would, without launching
+ * (host-only; usable without a GPU).  which: 0 = forward, 1 = backward. */
+int fa2_validate(const fa2_params* p, int which);
+
+const char* fa2_strerror(int code);
+int fa2_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FA2_H_ */

@@ -1,0 +1,204 @@
+// C ABI of libfa2_hip.so: argument validation and kernel dispatch.
+// Declarations and the reference call sites they replace: include/fa2.h.
+#include "../../include/fa2.h"
+
+#include <math.h>
+#include <string.h>
+
+#include "fa2_kernels.hpp"
+
+namespace {
+
+using fa2::KArgs;
+using fa2::KTensor;
+
+bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+int check_tensor(const fa2_tensor& t, bool required) {
+	if (!t.ptr) return required ? FA2_EINVAL_PTR : FA2_OK;
+	if (!aligned16(t.ptr)) return FA2_EINVAL_PTR;
+	// 16-byte vector access along D needs every row start 16-byte aligned
+	if (t.stride_b % 8 || t.stride_s % 8 || t.stride_h % 8) return FA2_EINVAL_STRIDE;
+	return FA2_OK;
+}
+
+int esize(int dtype) { return dtype == FA2_FP32 ? 4 : 2; }
+
+KTensor conv(const fa2_tensor& t) {
+	KTensor k;
+	k.ptr = (char*)t.ptr;
+	k.sb = t.stride_b * 2;
+	k.ss = t.stride_s * 2;
+	k.sh = t.stride_h * 2;
+	return k;
+}
+
+int validate(const fa2_params* p, int which) {
+	if (!p || p->struct_size < sizeof(fa2_params)) return FA2_EINVAL_STRUCT;
+	if (p->dtype != FA2_FP16 && p->dtype != FA2_BF16) return FA2_EINVAL_DTYPE;
+	if (p->B <= 0 || p->Sq <= 0 || p->Sk <= 0 || p->Hq <= 0 || p->Hkv <= 0 || p->D <= 0) return FA2_EINVAL_SHAPE;
+	if (p->Hq % p->Hkv) return FA2_EINVAL_HEADS;
+	if (p->D != 64 && p->D != 128 && p->D != 256) return FA2_EUNSUPPORTED;
+	if (!(p->p_drop >= 0.f && p->p_drop < 1.f)) return FA2_EINVAL_DROPOUT;
+	if (!isfinite(p->scale)) return FA2_EINVAL_SHAPE;
+	int rc;
+	if ((rc = check_tensor(p->q, true))) return rc;
+	if ((rc = check_tensor(p->k, true))) return rc;
+	if ((rc = check_tensor(p->v, true))) return rc;
+	if ((rc = check_tensor(p->o, true))) return rc;
+	if (!p->lse || ((uintptr_t)p->lse & 3)) return FA2_EINVAL_PTR;
+	if (p->bias) {
+		if (p->bias_dtype != FA2_FP16 && p->bias_dtype != FA2_BF16 && p->bias_dtype != FA2_FP32) return FA2_EINVAL_BIAS;
+		if (((uintptr_t)p->bias % esize(p->bias_dtype)) != 0) return FA2_EINVAL_BIAS;
+		if (p->bias_stride_b < 0 || p->bias_stride_h < 0 || p->bias_stride_m < p->Sk) return FA2_EINVAL_BIAS;
+	}
+	if (p->seqlens) {
+		if (p->bias || p->Sq != p->Sk) return FA2_EINVAL_MASK;
+		if ((uintptr_t)p->seqlens & 3) return FA2_EINVAL_PTR;
+	}
+	if (which == 1) {
+		if ((rc = check_tensor(p->dout, true))) return rc;
+		if ((rc = check_tensor(p->dq, true))) return rc;
+		if ((rc = check_tensor(p->dk, true))) return rc;
+		if ((rc = check_tensor(p->dv, true))) return rc;
+		size_t need = fa2_bwd_scratch_bytes(p);
+		if (!p->scratch || ((uintptr_t)p->scratch & 255) || p->scratch_bytes < need) return FA2_ESCRATCH;
+	}
+	return FA2_OK;
+}
+
+uint32_t drop_threshold(float p) {
+	double t = floor((double)p * 4294967296.0);
+	return t >= 4294967295.0 ? 0xFFFFFFFFu : (uint32_t)t;
+}
+
+void fill(const fa2_params* p, KArgs& a) {
+	memset(&a, 0, sizeof(a));
+	a.q = conv(p->q);
+	a.k = conv(p->k);
+	a.v = conv(p->v);
+	a.o = conv(p->o);
+	a.lse = p->lse;
+	a.bias = (const char*)p->bias;
+	if (p->bias) {
+		int es = esize(p->bias_dtype);
+		a.bias_sb = p->bias_stride_b * es;
+		a.bias_sh = p->bias_stride_h * es;
+		a.bias_sm = p->bias_stride_m * es;
+		a.bias_dtype = p->bias_dtype;
+		a.bias_group = p->bias_group ? 1 : 0;
+		int valign = es == 4 ? 16 : 8;
+		a.bias_vec4 = (((uintptr_t)p->bias % valign) == 0 && a.bias_sb % valign == 0 && a.bias_sh % valign == 0 &&
+		               a.bias_sm % valign == 0)
+		                  ? 1
+		                  : 0;
+	}
+	a.seqlens = p->seqlens;
+	a.B = p->B;
+	a.Sq = p->Sq;
+	a.Sk = p->Sk;
+	a.Hq = p->Hq;
+	a.Hkv = p->Hkv;
+	a.causal = p->causal ? 1 : 0;
+	a.scale = p->scale;
+	a.drop_k0 = (uint32_t)(p->seed & 0xFFFFFFFFull);
+	a.drop_k1 = (uint32_t)(p->seed >> 32);
+	a.drop_thr = drop_threshold(p->p_drop);
+	a.drop_inv_keep = 1.0f / (1.0f - p->p_drop);
+}
+
+}  // namespace
+
+namespace fa2 {
+
+hipError_t launch_fwd(int dtype, int D, bool bias, bool drop, KArgs& a, hipStream_t s) {
+	if (dtype == FA2_BF16) {
+		if (D == 64) return launch_fwd_bf16_64(bias, drop, a, s);
+		if (D == 128) return launch_fwd_bf16_128(bias, drop, a, s);
+		return launch_fwd_bf16_256(bias, drop, a, s);
+	}
+	if (D == 64) return launch_fwd_fp16_64(bias, drop, a, s);
+	if (D == 128) return launch_fwd_fp16_128(bias, drop, a, s);
+	return launch_fwd_fp16_256(bias, drop, a, s);
+}
+
+hipError_t launch_bwd(int dtype, int D, bool bias, bool drop, KArgs& a, hipStream_t s) {
+	if (dtype == FA2_BF16) {
+		if (D == 64) return launch_bwd_bf16_64(bias, drop, a, s);
+		if (D == 128) return launch_bwd_bf16_128(bias, drop, a, s);
+		return launch_bwd_bf16_256(bias, drop, a, s);
+	}
+	if (D == 64) return launch_bwd_fp16_64(bias, drop, a, s);
+	if (D == 128) return launch_bwd_fp16_128(bias, drop, a, s);
+	return launch_bwd_fp16_256(bias, drop, a, s);
+}
+
+}  // namespace fa2
+
+extern "C" {
+
+int fa2_validate(const fa2_params* p, int which) { return validate(p, which ? 1 : 0); }
+
+size_t fa2_bwd_scratch_bytes(const fa2_params* p) {
+	if (!p || p->struct_size < sizeof(fa2_params)) return 0;
+	if (p->B <= 0 || p->Hq <= 0 || p->Sq <= 0) return 0;
+	// delta [B, Hq, Sq] fp32, rounded up to 256 bytes
+	size_t n = (size_t)p->B * (size_t)p->Hq * (size_t)p->Sq * sizeof(float);
+	return (n + 255) & ~(size_t)255;
+}
+
+int fa2_fwd(const fa2_params* p, void* hip_stream) {
+	int rc = validate(p, 0);
+	if (rc) return rc;
+	KArgs a;
+	fill(p, a);
+	hipError_t e = fa2::launch_fwd(p->dtype, p->D, p->bias != nullptr, p->p_drop > 0.f, a, (hipStream_t)hip_stream);
+	return e == hipSuccess ? FA2_OK : FA2_EHIP;
+}
+
+int fa2_bwd(const fa2_params* p, void* hip_stream) {
+	int rc = validate(p, 1);
+	if (rc) return rc;
+	KArgs a;
+	fill(p, a);
+	a.dout = conv(p->dout);
+	a.dq = conv(p->dq);
+	a.dk = conv(p->dk);
+	a.dv = conv(p->dv);
+	a.delta = (float*)p->scratch;
+	hipError_t e = fa2::launch_bwd(p->dtype, p->D, p->bias != nullptr, p->p_drop > 0.f, a, (hipStream_t)hip_stream);
+	return e == hipSuccess ? FA2_OK : FA2_EHIP;
+}
+
+int fa2_dropout_mask(const fa2_params* p, uint8_t* keep, void* hip_stream) {
+	if (!p || p->struct_size < sizeof(fa2_params)) return FA2_EINVAL_STRUCT;
+	if (p->B <= 0 || p->Sq <= 0 || p->Sk <= 0 || p->Hq <= 0) return FA2_EINVAL_SHAPE;
+	if (!(p->p_drop >= 0.f && p->p_drop < 1.f)) return FA2_EINVAL_DROPOUT;
+	if (!keep) return FA2_EINVAL_PTR;
+	hipError_t e = fa2::launch_dropout_mask(keep, p->B, p->Hq, p->Sq, p->Sk, (uint32_t)(p->seed & 0xFFFFFFFFull),
+	                                        (uint32_t)(p->seed >> 32), drop_threshold(p->p_drop), (hipStream_t)hip_stream);
+	return e == hipSuccess ? FA2_OK : FA2_EHIP;
+}
+
+const char* fa2_strerror(int code) {
+	switch (code) {
+		case FA2_OK: return "ok";
+		case FA2_EINVAL_STRUCT: return "params is NULL or struct_size is smaller than sizeof(fa2_params)";
+		case FA2_EINVAL_DTYPE: return "Only support fp16 and bf16";
+		case FA2_EINVAL_SHAPE: return "dimensions must be positive and scale finite";
+		case FA2_EINVAL_HEADS: return "query heads must be divisible by key/value heads";
+		case FA2_EINVAL_PTR: return "required pointer is NULL or misaligned";
+		case FA2_EINVAL_STRIDE: return "batch/sequence/head strides must be multiples of 8 elements";
+		case FA2_EINVAL_DROPOUT: return "dropout probability must be in [0, 1)";
+		case FA2_EINVAL_BIAS: return "bias dtype or strides invalid";
+		case FA2_EINVAL_MASK: return "Attention mask is not supported along with attention bias or with QSeq != KSeq";
+		case FA2_EUNSUPPORTED: return "head dim must be 64, 128 or 256";
+		case FA2_ESCRATCH: return "backward scratch buffer missing, misaligned or too small";
+		case FA2_EHIP: return "HIP launch failed";
+		default: return "unknown error";
+	}
+}
+
+int fa2_version(void) { return 100; }
+
+}  // extern "C"

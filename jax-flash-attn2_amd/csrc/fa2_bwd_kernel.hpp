@@ -1,0 +1,584 @@
+// Backward kernels: delta pre-pass, dK/dV kernel, dQ kernel.  They take the
+// place of `_attn_bwd_preprocess` and `_attn_bwd` with its two roles
+// (jax_flash_attn2/flash_attention_triton/_backward_triton.py:79-147, 150-435,
+// 438-709, 712-945) and of the XLA sum over each KV group (:1156-1161).
+//
+// P is recomputed from the saved logsumexp.  With dropout, the same
+// position-keyed Philox mask as the forward is regenerated.
+//
+// dK/dV kernel: one workgroup = NW waves x 32 keys of one (batch, KV head);
+// K and V rows live in registers; Q and dO tiles of the r = Hq/Hkv query
+// heads of the group are streamed through LDS, so dK and dV accumulate over
+// the whole group in registers - no atomics and no per-q-head temporary.
+//   S  [q, kv] = Q K^T          A = Q from LDS,            B = K in registers
+//   dP [q, kv] = dO V^T         A = dO from LDS,           B = V in registers
+//   dV^T[d,kv] += dO^T P        A = dO, transposed LDS read, B = P  (S accumulator packed)
+//   dK^T[d,kv] += Q^T  dS       A = Q,  transposed LDS read, B = dS
+//
+// dQ kernel: one workgroup = one tile of query rows of one (batch, q-head),
+// K/V tiles streamed exactly as in the forward.
+//   S^T [kv, q] = K Q^T ; dP^T[kv, q] = V dO^T     (Q, dO in registers)
+//   dQ^T[d,  q] += K^T dS^T     A = K, transposed LDS read, B = dS^T packed
+#pragma once
+#include "fa2_common.hpp"
+#include "fa2_fwd_kernel.hpp"
+#include "fa2_kernels.hpp"
+
+namespace fa2 {
+
+// ---------------------------------------------------------------------------
+// delta[b,h,i] = sum_d O[b,i,h,d] * dO[b,i,h,d]     (HBM-bound; reads O and dO once)
+// ---------------------------------------------------------------------------
+template <typename T, int D>
+__global__ __launch_bounds__(256) void bwd_delta_kernel(const KArgs a) {
+	constexpr int TPR = D / 8;          // threads per row, 8 elements each
+	constexpr int RPB = 256 / TPR;      // rows per block
+	int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / TPR;
+	int part = threadIdx.x % TPR;
+	int64_t nrows = (int64_t)a.B * a.Sq * a.Hq;
+	float acc = 0.f;
+	int h = 0, b = 0, i = 0;
+	if (row < nrows) {
+		h = (int)(row % a.Hq);
+		int64_t r = row / a.Hq;
+		i = (int)(r % a.Sq);
+		b = (int)(r / a.Sq);
+		typename T::V8 o = *(const typename T::V8*)(a.o.ptr + b * a.o.sb + (int64_t)i * a.o.ss + (int64_t)h * a.o.sh + part * 16);
+		typename T::V8 d = *(const typename T::V8*)(a.dout.ptr + b * a.dout.sb + (int64_t)i * a.dout.ss + (int64_t)h * a.dout.sh + part * 16);
+#pragma unroll
+		for (int e = 0; e < 8; ++e) acc += (float)o[e] * (float)d[e];
+	}
+#pragma unroll
+	for (int sft = TPR / 2; sft >= 1; sft >>= 1) acc += __shfl_xor(acc, sft, 64);
+	if (row < nrows && part == 0) a.delta[((int64_t)b * a.Hq + h) * a.Sq + i] = acc;
+}
+
+// ---------------------------------------------------------------------------
+// dK / dV
+// ---------------------------------------------------------------------------
+template <typename T, int D, int NW, int QB, bool BIAS, bool DROP>
+__global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
+	typedef typename T::V8 V8;
+	constexpr int BN = NW * 32;     // keys per workgroup
+	constexpr int BMQ = QB * 32;    // query rows per streamed tile
+	constexpr int KS = D / 16;
+	constexpr int DB = D / 32;
+	constexpr int NT = NW * 64;
+	constexpr int TILE_BYTES = BMQ * D * 2;
+	constexpr int STAT_BYTES = BMQ * 4;
+
+	// Q[0] Q[1] dO[0] dO[1] | lse[0] lse[1] delta[0] delta[1]
+	__shared__ __attribute__((aligned(1024))) char smem[4 * TILE_BYTES + 4 * STAT_BYTES];
+	FA2_LDS char* lds = (FA2_LDS char*)smem;
+	FA2_LDS char* stat = lds + 4 * TILE_BYTES;
+
+	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+	const int g = lane >> 5, c = lane & 31;
+	const int r = a.Hq / a.Hkv;
+
+	// blockIdx.x -> (key tile, kv head, batch); key tiles of one (b, kv head) stay on one XCD
+	int nt, hk, b;
+	{
+		int id = blockIdx.x;
+		int per_group = a.mtiles;
+		int grp, within;
+		if (a.xcd_remap) {
+			int xcd = id & 7, j = id >> 3;
+			grp = (j / per_group) * 8 + xcd;
+			within = j % per_group;
+		} else {
+			grp = id / per_group;
+			within = id % per_group;
+		}
+		hk = grp % a.Hkv;
+		b = grp / a.Hkv;
+		nt = within;  // early key tiles see the most query rows under a causal mask: first
+	}
+
+	int sq_eff = a.Sq, sk_eff = a.Sk;
+	if (a.seqlens) {
+		int len = a.seqlens[b];
+		len = len < 0 ? 0 : (len > a.Sk ? a.Sk : len);
+		sq_eff = len < a.Sq ? len : a.Sq;
+		sk_eff = len;
+	}
+	const int off = sk_eff - sq_eff;
+	const int n0 = nt * BN;
+	const int wn0 = n0 + 32 * w;
+	const int jcol = wn0 + c;  // this lane's key
+
+	// K, V rows of this lane's key as B operands: lane holds X[jcol][16ks + 8g .. +7]
+	V8 kf[KS], vf[KS];
+	{
+		int j = jcol < a.Sk ? jcol : a.Sk - 1;
+		const char* kp = a.k.ptr + (int64_t)b * a.k.sb + (int64_t)hk * a.k.sh + (int64_t)j * a.k.ss + g * 16;
+		const char* vp = a.v.ptr + (int64_t)b * a.v.sb + (int64_t)hk * a.v.sh + (int64_t)j * a.v.ss + g * 16;
+#pragma unroll
+		for (int ks = 0; ks < KS; ++ks) {
+			kf[ks] = *(const V8*)(kp + ks * 32);
+			vf[ks] = *(const V8*)(vp + ks * 32);
+		}
+	}
+
+	f32x16 dk[DB], dv[DB];
+#pragma unroll
+	for (int db = 0; db < DB; ++db)
+#pragma unroll
+		for (int i = 0; i < 16; ++i) dk[db][i] = dv[db][i] = 0.f;
+
+	// query tiles that see at least one key of this workgroup
+	int q_lo = 0;
+	if (a.causal) {
+		int first = n0 - off;  // first row allowed to see key n0
+		q_lo = first > 0 ? first / BMQ : 0;
+	}
+	int q_hi = (sq_eff + BMQ - 1) / BMQ;  // exclusive
+	if (n0 >= sk_eff) q_hi = q_lo;
+	const int nq = q_hi > q_lo ? q_hi - q_lo : 0;
+	const int steps = nq * r;
+
+	const float c1 = BIAS ? a.scale : a.scale * kLog2e;
+
+	auto issue_tile = [&](int step, int buf) {
+		int hq = hk * r + step / nq;
+		int m0 = (q_lo + step % nq) * BMQ;
+		int rows = a.Sq - m0 < BMQ ? a.Sq - m0 : BMQ;
+		const char* qb_ = a.q.ptr + (int64_t)b * a.q.sb + (int64_t)hq * a.q.sh + (int64_t)m0 * a.q.ss;
+		const char* db_ = a.dout.ptr + (int64_t)b * a.dout.sb + (int64_t)hq * a.dout.sh + (int64_t)m0 * a.dout.ss;
+		tile_load_async<D, BMQ, NT>(lds + buf * TILE_BYTES, qb_, a.q.ss, rows, tid);
+		tile_load_async<D, BMQ, NT>(lds + (2 + buf) * TILE_BYTES, db_, a.dout.ss, rows, tid);
+	};
+	// per-row statistics of a tile: thread t < BMQ fetches lse, t in [BMQ, 2 BMQ) fetches delta
+	auto fetch_stat = [&](int step) -> float {
+		float x = 0.f;
+		if (tid < 2 * BMQ) {
+			int hq = hk * r + step / nq;
+			int m0 = (q_lo + step % nq) * BMQ;
+			int i = m0 + (tid % BMQ);
+			i = i < a.Sq ? i : a.Sq - 1;
+			int64_t idx = ((int64_t)b * a.Hq + hq) * a.Sq + i;
+			if (tid < BMQ) {
+				x = a.lse[idx];
+				if constexpr (!BIAS) x *= kLog2e;
+			} else {
+				x = a.delta[idx];
+			}
+		}
+		return x;
+	};
+	auto store_stat = [&](float x, int buf) {
+		if (tid < 2 * BMQ) {
+			int which = tid / BMQ;
+			*(FA2_LDS float*)(stat + (2 * which + buf) * STAT_BYTES + (tid % BMQ) * 4) = x;
+		}
+	};
+
+	if (steps > 0) {
+		issue_tile(0, 0);
+		store_stat(fetch_stat(0), 0);
+	}
+
+	for (int step = 0; step < steps; ++step) {
+		const int buf = step & 1;
+		wait_async_loads();
+		__syncthreads();
+		float next_stat = 0.f;
+		const bool has_next = step + 1 < steps;
+		if (has_next) {
+			issue_tile(step + 1, buf ^ 1);
+			next_stat = fetch_stat(step + 1);
+		}
+		const int hq = hk * r + step / nq;
+		const int m0 = (q_lo + step % nq) * BMQ;
+		// wave-uniform: any work / any masking for (rows m0.., keys wn0..)?
+		int last_row = m0 + BMQ - 1 < sq_eff - 1 ? m0 + BMQ - 1 : sq_eff - 1;
+		bool skip = wn0 >= sk_eff || (a.causal && wn0 > last_row + off);
+		if (!skip) {
+			const bool need_mask = (m0 + BMQ > sq_eff) || (wn0 + 32 > sk_eff) || (a.causal && wn0 + 31 > m0 + off);
+			const FA2_LDS char* qt = lds + buf * TILE_BYTES;
+			const FA2_LDS char* dot = lds + (2 + buf) * TILE_BYTES;
+			const FA2_LDS char* lse_s = stat + buf * STAT_BYTES;
+			const FA2_LDS char* del_s = stat + (2 + buf) * STAT_BYTES;
+			const char* bias_base = nullptr;
+			if constexpr (BIAS) {
+				int hb = a.bias_group ? hk : hq;
+				int jc = jcol < a.Sk ? jcol : a.Sk - 1;
+				int es = a.bias_dtype == 3 ? 4 : 2;
+				bias_base = a.bias + (int64_t)b * a.bias_sb + (int64_t)hb * a.bias_sh + (int64_t)jc * es;
+			}
+#pragma unroll
+			for (int qb = 0; qb < QB; ++qb) {
+				// bias column for this lane's key, 16 rows
+				float bv[BIAS ? 16 : 1];
+				if constexpr (BIAS) {
+#pragma unroll
+					for (int i = 0; i < 16; ++i) {
+						int row = m0 + 32 * qb + 8 * (i >> 2) + 4 * g + (i & 3);
+						row = row < a.Sq ? row : a.Sq - 1;
+						const char* pp = bias_base + (int64_t)row * a.bias_sm;
+						bv[i] = a.bias_dtype == 3 ? *(const float*)pp
+						        : a.bias_dtype == 2 ? (float)*(const __bf16*)pp
+						                            : (float)*(const _Float16*)pp;
+					}
+				}
+				f32x16 s, dp;
+#pragma unroll
+				for (int i = 0; i < 16; ++i) s[i] = dp[i] = 0.f;
+#pragma unroll
+				for (int ks = 0; ks < KS; ++ks) {
+					V8 qa = lds_frag<T, D>(qt, 32 * qb, ks, lane);
+					s = mfma32(qa, kf[ks], s);
+				}
+#pragma unroll
+				for (int ks = 0; ks < KS; ++ks) {
+					V8 da = lds_frag<T, D>(dot, 32 * qb, ks, lane);
+					dp = mfma32(da, vf[ks], dp);
+				}
+				f32x4 lse4[4], del4[4];
+#pragma unroll
+				for (int aa = 0; aa < 4; ++aa) {
+					lse4[aa] = *(const FA2_LDS f32x4*)(lse_s + (32 * qb + 8 * aa + 4 * g) * 4);
+					del4[aa] = *(const FA2_LDS f32x4*)(del_s + (32 * qb + 8 * aa + 4 * g) * 4);
+				}
+				f32x16 pd;  // P after dropout (feeds dV); s becomes dS (feeds dK)
+#pragma unroll
+				for (int i = 0; i < 16; ++i) {
+					int row = m0 + 32 * qb + 8 * (i >> 2) + 4 * g + (i & 3);
+					float lse = lse4[i >> 2][i & 3], del = del4[i >> 2][i & 3];
+					float p;
+					if constexpr (BIAS)
+						p = exp2_fast((__builtin_fmaf(s[i], c1, bv[i]) - lse) * kLog2e);
+					else
+						p = exp2_fast(__builtin_fmaf(s[i], c1, -lse));
+					if (need_mask) {
+						bool ok = row < sq_eff && jcol < sk_eff && (!a.causal || jcol <= row + off);
+						p = ok ? p : 0.f;
+					}
+					float pdrop = p, dpe = dp[i];
+					if constexpr (DROP) {
+						u32x4 rnd = philox4x32_10((uint32_t)(jcol >> 2), (uint32_t)row, (uint32_t)hq, (uint32_t)b, a.drop_k0, a.drop_k1);
+						uint32_t word = rnd[0];
+						word = (jcol & 3) == 1 ? rnd[1] : word;
+						word = (jcol & 3) == 2 ? rnd[2] : word;
+						word = (jcol & 3) == 3 ? rnd[3] : word;
+						bool keep = word >= a.drop_thr;
+						pdrop = keep ? p : 0.f;
+						dpe = keep ? dpe * a.drop_inv_keep : 0.f;
+					}
+					pd[i] = pdrop;
+					s[i] = p * (dpe - del);
+				}
+				// dV^T += dO^T P ; dK^T += Q^T dS   (k runs over the tile's 32 rows, two steps of 16)
+#pragma unroll
+				for (int hf = 0; hf < 2; ++hf) {
+					V8 pb = pack8<T>(pd[8 * hf + 0], pd[8 * hf + 1], pd[8 * hf + 2], pd[8 * hf + 3], pd[8 * hf + 4], pd[8 * hf + 5],
+					                 pd[8 * hf + 6], pd[8 * hf + 7]);
+					V8 sb = pack8<T>(s[8 * hf + 0], s[8 * hf + 1], s[8 * hf + 2], s[8 * hf + 3], s[8 * hf + 4], s[8 * hf + 5],
+					                 s[8 * hf + 6], s[8 * hf + 7]);
+#pragma unroll
+					for (int db = 0; db < DB; ++db) {
+						V8 dot_a = lds_frag_tr<T, D>(dot, 32 * qb + 16 * hf, 32 * db, lane);
+						dv[db] = mfma32(dot_a, pb, dv[db]);
+						V8 qt_a = lds_frag_tr<T, D>(qt, 32 * qb + 16 * hf, 32 * db, lane);
+						dk[db] = mfma32(qt_a, sb, dk[db]);
+					}
+				}
+			}
+		}
+		if (has_next) store_stat(next_stat, buf ^ 1);
+	}
+
+	// epilogue: lane owns key jcol, four consecutive d per store
+	if (jcol < a.Sk) {
+		char* dkp = a.dk.ptr + (int64_t)b * a.dk.sb + (int64_t)hk * a.dk.sh + (int64_t)jcol * a.dk.ss;
+		char* dvp = a.dv.ptr + (int64_t)b * a.dv.sb + (int64_t)hk * a.dv.sh + (int64_t)jcol * a.dv.ss;
+		const float ks_ = a.scale;
+		const float vs_ = DROP ? a.drop_inv_keep : 1.f;
+#pragma unroll
+		for (int db = 0; db < DB; ++db)
+#pragma unroll
+			for (int aa = 0; aa < 4; ++aa) {
+				int d0 = 32 * db + 8 * aa + 4 * g;
+				u32x2 pk = {pack2<typename T::V2>(dk[db][4 * aa] * ks_, dk[db][4 * aa + 1] * ks_),
+				            pack2<typename T::V2>(dk[db][4 * aa + 2] * ks_, dk[db][4 * aa + 3] * ks_)};
+				*(u32x2*)(dkp + d0 * 2) = pk;
+				u32x2 pv = {pack2<typename T::V2>(dv[db][4 * aa] * vs_, dv[db][4 * aa + 1] * vs_),
+				            pack2<typename T::V2>(dv[db][4 * aa + 2] * vs_, dv[db][4 * aa + 3] * vs_)};
+				*(u32x2*)(dvp + d0 * 2) = pv;
+			}
+	}
+}
+
+// ---------------------------------------------------------------------------
+// dQ
+// ---------------------------------------------------------------------------
+template <typename T, int D, int NW, int QB, bool BIAS, bool DROP>
+__global__ __launch_bounds__(NW * 64) void bwd_dq_kernel(const KArgs a) {
+	typedef typename T::V8 V8;
+	constexpr int BM = NW * QB * 32;
+	constexpr int BN = kFwdBN;
+	constexpr int KB = BN / 32;
+	constexpr int KS = D / 16;
+	constexpr int DB = D / 32;
+	constexpr int NT = NW * 64;
+	constexpr int TILE_BYTES = BN * D * 2;
+
+	__shared__ __attribute__((aligned(1024))) char smem[4 * TILE_BYTES];
+	FA2_LDS char* lds = (FA2_LDS char*)smem;
+
+	int mt, h, b;
+	decode_block(a, mt, h, b);
+	const int hk = h / (a.Hq / a.Hkv);
+	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+	const int g = lane >> 5, c = lane & 31;
+
+	int sq_eff = a.Sq, sk_eff = a.Sk;
+	if (a.seqlens) {
+		int len = a.seqlens[b];
+		len = len < 0 ? 0 : (len > a.Sk ? a.Sk : len);
+		sq_eff = len < a.Sq ? len : a.Sq;
+		sk_eff = len;
+	}
+	const int off = sk_eff - sq_eff;
+	const int m0 = mt * BM;
+	const int wm0 = m0 + w * (QB * 32);
+
+	int kv_end = sk_eff;
+	if (a.causal) {
+		int last_row = (m0 + BM - 1 < sq_eff - 1) ? m0 + BM - 1 : sq_eff - 1;
+		int e = last_row + off + 1;
+		kv_end = e < kv_end ? e : kv_end;
+	}
+	if (m0 >= sq_eff) kv_end = 0;
+	const int ntiles = kv_end > 0 ? (kv_end + BN - 1) / BN : 0;
+
+	int jmax[QB], qrow[QB];
+	float lse_r[QB], del_r[QB];
+#pragma unroll
+	for (int qb = 0; qb < QB; ++qb) {
+		int i = wm0 + 32 * qb + c;
+		qrow[qb] = i;
+		int jm = sk_eff - 1;
+		if (a.causal) jm = (i + off < jm) ? i + off : jm;
+		if (i >= sq_eff) jm = -1;
+		jmax[qb] = jm;
+		int ic = i < a.Sq ? i : a.Sq - 1;
+		int64_t idx = ((int64_t)b * a.Hq + h) * a.Sq + ic;
+		float l = a.lse[idx];
+		// rows without any allowed key carry lse = -inf; their P is forced to 0 by the mask
+		lse_r[qb] = BIAS ? l : l * kLog2e;
+		del_r[qb] = a.delta[idx];
+	}
+	int wave_jmin, wave_jmax;
+	{
+		int first = wm0, last = wm0 + QB * 32 - 1;
+		if (first >= sq_eff) {
+			wave_jmin = wave_jmax = -1;
+		} else {
+			wave_jmax = sk_eff - 1;
+			wave_jmin = sk_eff - 1;
+			int lastv = last < sq_eff - 1 ? last : sq_eff - 1;
+			if (a.causal) {
+				wave_jmax = (lastv + off < wave_jmax) ? lastv + off : wave_jmax;
+				wave_jmin = (first + off < wave_jmin) ? first + off : wave_jmin;
+			}
+			if (last >= sq_eff) wave_jmin = -1;
+		}
+	}
+
+	const char* kbase = a.k.ptr + (int64_t)b * a.k.sb + (int64_t)hk * a.k.sh;
+	const char* vbase = a.v.ptr + (int64_t)b * a.v.sb + (int64_t)hk * a.v.sh;
+	if (ntiles > 0) {
+		int rows = sk_eff < BN ? sk_eff : BN;
+		tile_load_async<D, BN, NT>(lds, kbase, a.k.ss, rows, tid);
+		tile_load_async<D, BN, NT>(lds + 2 * TILE_BYTES, vbase, a.v.ss, rows, tid);
+	}
+
+	V8 qf[QB][KS], dof[QB][KS];
+	{
+		const char* qbase = a.q.ptr + (int64_t)b * a.q.sb + (int64_t)h * a.q.sh;
+		const char* dbase = a.dout.ptr + (int64_t)b * a.dout.sb + (int64_t)h * a.dout.sh;
+#pragma unroll
+		for (int qb = 0; qb < QB; ++qb) {
+			int i = qrow[qb] < a.Sq ? qrow[qb] : a.Sq - 1;
+			const char* rp = qbase + (int64_t)i * a.q.ss + g * 16;
+			const char* dp_ = dbase + (int64_t)i * a.dout.ss + g * 16;
+#pragma unroll
+			for (int ks = 0; ks < KS; ++ks) {
+				qf[qb][ks] = *(const V8*)(rp + ks * 32);
+				dof[qb][ks] = *(const V8*)(dp_ + ks * 32);
+			}
+		}
+	}
+
+	f32x16 dq[QB][DB];
+#pragma unroll
+	for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+		for (int db = 0; db < DB; ++db)
+#pragma unroll
+			for (int i = 0; i < 16; ++i) dq[qb][db][i] = 0.f;
+
+	const float c1 = BIAS ? a.scale : a.scale * kLog2e;
+	const char* bias_base = nullptr;
+	if constexpr (BIAS) {
+		int hb = a.bias_group ? hk : h;
+		bias_base = a.bias + (int64_t)b * a.bias_sb + (int64_t)hb * a.bias_sh;
+	}
+
+	for (int t = 0; t < ntiles; ++t) {
+		const int n0 = t * BN;
+		const int buf = t & 1;
+		wait_async_loads();
+		__syncthreads();
+		if (t + 1 < ntiles) {
+			int n1 = n0 + BN;
+			int rows = sk_eff - n1 < BN ? sk_eff - n1 : BN;
+			tile_load_async<D, BN, NT>(lds + (buf ^ 1) * TILE_BYTES, kbase + (int64_t)n1 * a.k.ss, a.k.ss, rows, tid);
+			tile_load_async<D, BN, NT>(lds + (2 + (buf ^ 1)) * TILE_BYTES, vbase + (int64_t)n1 * a.v.ss, a.v.ss, rows, tid);
+		}
+		if (n0 > wave_jmax) continue;
+		const bool need_mask = n0 + BN - 1 > wave_jmin;
+		const FA2_LDS char* kt = lds + buf * TILE_BYTES;
+		const FA2_LDS char* vt = lds + (2 + buf) * TILE_BYTES;
+
+#pragma unroll
+		for (int kb = 0; kb < KB; ++kb) {
+			f32x4 bv[BIAS ? QB : 1][4];
+			if constexpr (BIAS) {
+#pragma unroll
+				for (int qb = 0; qb < QB; ++qb) {
+					int i = qrow[qb] < a.Sq ? qrow[qb] : a.Sq - 1;
+					const char* rowp = bias_base + (int64_t)i * a.bias_sm;
+#pragma unroll
+					for (int aa = 0; aa < 4; ++aa)
+						bv[qb][aa] = load_bias4(rowp, n0 + 32 * kb + 8 * aa + 4 * g, a.bias_dtype, a.bias_vec4, a.Sk);
+				}
+			}
+			f32x16 s[QB], dp[QB];
+#pragma unroll
+			for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+				for (int i = 0; i < 16; ++i) s[qb][i] = dp[qb][i] = 0.f;
+#pragma unroll
+			for (int ks = 0; ks < KS; ++ks) {
+				V8 ka = lds_frag<T, D>(kt, 32 * kb, ks, lane);
+#pragma unroll
+				for (int qb = 0; qb < QB; ++qb) s[qb] = mfma32(ka, qf[qb][ks], s[qb]);
+			}
+#pragma unroll
+			for (int ks = 0; ks < KS; ++ks) {
+				V8 va = lds_frag<T, D>(vt, 32 * kb, ks, lane);
+#pragma unroll
+				for (int qb = 0; qb < QB; ++qb) dp[qb] = mfma32(va, dof[qb][ks], dp[qb]);
+			}
+			V8 dsf[QB][2];
+#pragma unroll
+			for (int qb = 0; qb < QB; ++qb) {
+#pragma unroll
+				for (int aa = 0; aa < 4; ++aa) {
+					u32x4 rnd;
+					if constexpr (DROP) {
+						int j4 = (n0 + 32 * kb + 8 * aa + 4 * g) >> 2;
+						rnd = philox4x32_10((uint32_t)j4, (uint32_t)qrow[qb], (uint32_t)h, (uint32_t)b, a.drop_k0, a.drop_k1);
+					}
+#pragma unroll
+					for (int e = 0; e < 4; ++e) {
+						int i = 4 * aa + e;
+						float p;
+						if constexpr (BIAS)
+							p = exp2_fast((__builtin_fmaf(s[qb][i], c1, bv[qb][aa][e]) - lse_r[qb]) * kLog2e);
+						else
+							p = exp2_fast(__builtin_fmaf(s[qb][i], c1, -lse_r[qb]));
+						if (need_mask) {
+							int j = n0 + 32 * kb + 8 * aa + 4 * g + e;
+							p = j <= jmax[qb] ? p : 0.f;
+						}
+						float dpe = dp[qb][i];
+						if constexpr (DROP) dpe = rnd[e] >= a.drop_thr ? dpe * a.drop_inv_keep : 0.f;
+						s[qb][i] = p * (dpe - del_r[qb]);
+					}
+				}
+#pragma unroll
+				for (int hf = 0; hf < 2; ++hf) {
+					const f32x16& x = s[qb];
+					dsf[qb][hf] = pack8<T>(x[8 * hf + 0], x[8 * hf + 1], x[8 * hf + 2], x[8 * hf + 3], x[8 * hf + 4], x[8 * hf + 5],
+					                       x[8 * hf + 6], x[8 * hf + 7]);
+				}
+			}
+			// dQ^T += K^T dS^T
+#pragma unroll
+			for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+				for (int db = 0; db < DB; ++db) {
+					V8 kta = lds_frag_tr<T, D>(kt, 32 * kb + 16 * hf, 32 * db, lane);
+#pragma unroll
+					for (int qb = 0; qb < QB; ++qb) dq[qb][db] = mfma32(kta, dsf[qb][hf], dq[qb][db]);
+				}
+		}
+	}
+
+	char* obase = a.dq.ptr + (int64_t)b * a.dq.sb + (int64_t)h * a.dq.sh;
+#pragma unroll
+	for (int qb = 0; qb < QB; ++qb) {
+		int i = qrow[qb];
+		if (i < a.Sq) {
+			char* rp = obase + (int64_t)i * a.dq.ss;
+			const float sc = a.scale;
+#pragma unroll
+			for (int db = 0; db < DB; ++db)
+#pragma unroll
+				for (int aa = 0; aa < 4; ++aa) {
+					const f32x16& x = dq[qb][db];
+					u32x2 pk = {pack2<typename T::V2>(x[4 * aa] * sc, x[4 * aa + 1] * sc),
+					            pack2<typename T::V2>(x[4 * aa + 2] * sc, x[4 * aa + 3] * sc)};
+					*(u32x2*)(rp + (32 * db + 8 * aa + 4 * g) * 2) = pk;
+				}
+		}
+	}
+}
+
+template <typename T, int D>
+struct BwdCfg {
+	// dK/dV: 4 waves x 32 keys; query rows streamed 64 (32 for D = 256) at a time
+	static constexpr int KV_NW = 4;
+	static constexpr int KV_QB = D <= 128 ? 2 : 1;
+	static constexpr int KV_BN = KV_NW * 32;
+	// dQ: 4 waves x QB x 32 rows
+	static constexpr int DQ_NW = 4;
+	static constexpr int DQ_QB = D <= 64 ? 2 : 1;
+	static constexpr int DQ_BM = DQ_NW * DQ_QB * 32;
+};
+
+template <typename T, int D, bool BIAS, bool DROP>
+hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
+	typedef BwdCfg<T, D> C;
+	int groups = a.B * a.Hkv;
+	a.xcd_remap = (groups % 8 == 0) ? 1 : 0;
+	{
+		int64_t nrows = (int64_t)a.B * a.Sq * a.Hq;
+		constexpr int RPB = 256 / (D / 8);
+		hipLaunchKernelGGL((bwd_delta_kernel<T, D>), dim3((unsigned)((nrows + RPB - 1) / RPB)), dim3(256), 0, s, a);
+	}
+	{
+		a.mtiles = (a.Sk + C::KV_BN - 1) / C::KV_BN;
+		dim3 grid((unsigned)(a.mtiles * a.B * a.Hkv)), block(C::KV_NW * 64);
+		hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, C::KV_NW, C::KV_QB, BIAS, DROP>), grid, block, 0, s, a);
+	}
+	{
+		a.mtiles = (a.Sq + C::DQ_BM - 1) / C::DQ_BM;
+		dim3 grid((unsigned)(a.mtiles * a.B * a.Hq)), block(C::DQ_NW * 64);
+		hipLaunchKernelGGL((bwd_dq_kernel<T, D, C::DQ_NW, C::DQ_QB, BIAS, DROP>), grid, block, 0, s, a);
+	}
+	return hipGetLastError();
+}
+
+template <typename T, int D>
+hipError_t launch_bwd_t(bool bias, bool drop, KArgs& a, hipStream_t s) {
+	if (bias && drop) return launch_bwd_v<T, D, true, true>(a, s);
+	if (bias) return launch_bwd_v<T, D, true, false>(a, s);
+	if (drop) return launch_bwd_v<T, D, false, true>(a, s);
+	return launch_bwd_v<T, D, false, false>(a, s);
+}
+
+}  // namespace fa2

@@ -1,0 +1,188 @@
+// Device-side building blocks shared by the forward and backward kernels:
+// element types, MFMA wrappers, swizzled LDS tiles (plain and transposed
+// fragment reads), direct global->LDS tile copies, Philox dropout.
+// gfx950 (CDNA4) only.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fa2 {
+
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(4))) _Float16 f16x4;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+#define FA2_DEV __device__ __forceinline__
+#define FA2_LDS __attribute__((address_space(3)))
+#define FA2_GLB __attribute__((address_space(1)))
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// Element traits: E = storage element, V8/V4/V2 = vectors of it.
+struct BF16 {
+	typedef __bf16 E;
+	typedef bf16x8 V8;
+	typedef bf16x4 V4;
+	typedef bf16x2 V2;
+};
+struct FP16 {
+	typedef _Float16 E;
+	typedef f16x8 V8;
+	typedef f16x4 V4;
+	typedef f16x2 V2;
+};
+
+// D[32x32] += A[32x16] * B[16x32].  Lane l supplies A[row l%32][k 8*(l/32)..+7]
+// and B[k 8*(l/32)..+7][col l%32]; it receives D[row 8*(i/4)+4*(l/32)+i%4][col l%32]
+// in element i of the accumulator.
+FA2_DEV f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+	return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+FA2_DEV f32x16 mfma32(f16x8 a, f16x8 b, f32x16 c) {
+	return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+
+template <typename V2>
+FA2_DEV uint32_t pack2(float a, float b) {
+	f32x2 f = {a, b};
+	V2 h = __builtin_convertvector(f, V2);
+	return __builtin_bit_cast(uint32_t, h);
+}
+
+// Eight fp32 -> one 8-element MFMA operand.
+template <typename T>
+FA2_DEV typename T::V8 pack8(float x0, float x1, float x2, float x3, float x4, float x5, float x6, float x7) {
+	u32x4 u = {pack2<typename T::V2>(x0, x1), pack2<typename T::V2>(x2, x3), pack2<typename T::V2>(x4, x5),
+	           pack2<typename T::V2>(x6, x7)};
+	return __builtin_bit_cast(typename T::V8, u);
+}
+
+FA2_DEV float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
+FA2_DEV float log2_fast(float x) { return __builtin_amdgcn_logf(x); }
+
+// max of the values held by lane l and lane l^32
+FA2_DEV float pair_max(float x) {
+	auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(int, x), __builtin_bit_cast(int, x), false, false);
+	return __builtin_fmaxf(__builtin_bit_cast(float, (int)r[0]), __builtin_bit_cast(float, (int)r[1]));
+}
+FA2_DEV float pair_sum(float x) {
+	auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(int, x), __builtin_bit_cast(int, x), false, false);
+	return __builtin_bit_cast(float, (int)r[0]) + __builtin_bit_cast(float, (int)r[1]);
+}
+
+// ---------------------------------------------------------------------------
+// LDS tiles.  A tile is ROWS x D elements, row-major, 16-byte chunks XOR
+// swizzled inside each row so that (a) sixteen lanes reading the same chunk of
+// sixteen consecutive rows and (b) the four-row groups of a transposed read
+// fall on distinct banks.
+// ---------------------------------------------------------------------------
+template <int D>
+FA2_DEV int swz(int row) {
+	if constexpr (D >= 128)
+		return ((row & 3) << 2) | ((row >> 2) & 3);
+	else
+		return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
+}
+
+// byte offset of 16-byte chunk `chunk` of row `row`
+template <int D>
+FA2_DEV int tile_off(int row, int chunk) {
+	return row * (D * 2) + ((chunk ^ swz<D>(row)) << 4);
+}
+
+// Fragment for the operand whose 32 rows/cols are tile rows and whose MFMA k
+// runs along D: lane l gets tile[row0 + l%32][16*ks + 8*(l/32) .. +7].
+template <typename T, int D>
+FA2_DEV typename T::V8 lds_frag(const FA2_LDS char* tile, int row0, int ks, int lane) {
+	int row = row0 + (lane & 31);
+	int chunk = 2 * ks + (lane >> 5);
+	return *(const FA2_LDS typename T::V8*)(tile + tile_off<D>(row, chunk));
+}
+
+// Transposed fragment: the operand's 32 rows/cols run along D (col0..col0+31)
+// and its MFMA k runs along tile rows.  k-slot (g = l/32, j) is tile row
+// row0 + 4g + j for j < 4 and row0 + 8 + 4g + (j-4) for j >= 4, which is the
+// order in which a 32x32 accumulator holds its rows - so an accumulator
+// packed to 16 bits is directly the other operand.
+// Built from two ds_read_b64_tr_b16: inside a block of 16 lanes, lane i
+// receives element i%4 of the 8-byte rows fetched by lanes 4j + i/4, j=0..3.
+template <typename T, int D>
+FA2_DEV typename T::V8 lds_frag_tr(const FA2_LDS char* tile, int row0, int col0, int lane) {
+	int i16 = lane & 15;
+	int g = lane >> 5;
+	int row = row0 + 4 * g + (i16 >> 2);
+	int col = col0 + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
+	typedef __attribute__((__vector_size__(4 * sizeof(short)))) short v4s;
+	const FA2_LDS char* p0 = tile + tile_off<D>(row, col >> 3) + ((col & 4) << 1);
+	const FA2_LDS char* p1 = tile + tile_off<D>(row + 8, col >> 3) + ((col & 4) << 1);
+	v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FA2_LDS v4s*)p0);
+	v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FA2_LDS v4s*)p1);
+	typedef __attribute__((__vector_size__(8 * sizeof(short)))) short v8s;
+	v8s both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+	return __builtin_bit_cast(typename T::V8, both);
+}
+
+// Copy a ROWS x D tile from global memory (row stride `stride` elements) into
+// a swizzled LDS tile without passing through registers.  Each wave-level
+// instruction moves 64 x 16 bytes; lane i lands at LDS slot base + i, so the
+// swizzle is applied by choosing which global chunk each lane fetches.  Rows
+// at or beyond `rows_valid` are fetched from the last valid row instead (the
+// caller masks their scores), so no lane reads out of bounds.
+template <int D, int ROWS, int NTHREADS>
+FA2_DEV void tile_load_async(FA2_LDS char* tile, const char* gbase, int64_t stride_bytes, int rows_valid, int tid) {
+	constexpr int CPR = D / 8;  // 16-byte chunks per row
+	constexpr int TOTAL = ROWS * CPR;
+	static_assert(TOTAL % NTHREADS == 0, "tile must divide over the workgroup");
+	int wave_base = (tid >> 6) << 6;
+	int lane = tid & 63;
+#pragma unroll
+	for (int it = 0; it < TOTAL / NTHREADS; ++it) {
+		int slot0 = it * NTHREADS + wave_base;  // wave-uniform
+		int slot = slot0 + lane;
+		int row = slot / CPR;
+		int pchunk = slot % CPR;
+		int chunk = pchunk ^ swz<D>(row);
+		int grow = row < rows_valid ? row : rows_valid - 1;
+		const char* src = gbase + (int64_t)grow * stride_bytes + (chunk << 4);
+		__builtin_amdgcn_global_load_lds((const FA2_GLB void*)src, (FA2_LDS void*)(tile + slot0 * 16), 16, 0, 0);
+	}
+}
+
+FA2_DEV void wait_async_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// ---------------------------------------------------------------------------
+// Philox-4x32-10.  counter = (j >> 2, i, h, b), key = (seed lo, seed hi);
+// element (i, j) uses word j & 3 and is kept iff word >= threshold.
+// ---------------------------------------------------------------------------
+FA2_DEV u32x4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1) {
+#pragma unroll
+	for (int r = 0; r < 10; ++r) {
+		uint32_t hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
+		uint32_t hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+		uint32_t n0 = hi1 ^ c1 ^ k0, n2 = hi0 ^ c3 ^ k1;
+		c0 = n0;
+		c1 = lo1;
+		c2 = n2;
+		c3 = lo0;
+		k0 += 0x9E3779B9u;
+		k1 += 0xBB67AE85u;
+	}
+	u32x4 out = {c0, c1, c2, c3};
+	return out;
+}
+
+struct Dropout {
+	uint32_t k0, k1, thr;
+	float inv_keep;  // 1 / (1 - p)
+};
+
+}  // namespace fa2

@@ -1,0 +1,370 @@
+// Forward kernel: O = softmax(scale Q K^T + bias, masked) V, plus the row
+// logsumexp.  Takes the place of `_attn_fwd` / `_attn_fwd_inner`
+// (jax_flash_attn2/flash_attention_triton/_forward_triton.py:60-164, 213-459).
+//
+// One workgroup = NW waves = one tile of BM = NW*QB*32 query rows of one
+// (batch, q-head).  K/V tiles of BN = 64 keys are streamed through a double
+// buffer in LDS by direct global->LDS loads.  Everything is computed
+// transposed so that no intermediate ever leaves registers:
+//   S^T[kv, q] = K[kv, :] . Q[q, :]      A = K fragment from LDS, B = Q in registers
+//   O^T[d,  q] = V^T[d, kv] . P^T[kv, q] A = V through transposed LDS reads,
+//                                        B = P^T = the S^T accumulator, packed to 16 bits
+// In both accumulators a lane owns ONE query row (column l%32), so the online
+// softmax needs only in-lane reductions plus one exchange with lane l^32, and
+// rescaling O is a multiply by a per-lane scalar.
+#pragma once
+#include "fa2_common.hpp"
+#include "fa2_kernels.hpp"
+
+namespace fa2 {
+
+constexpr int kFwdBN = 64;
+
+// blockIdx.x -> (row tile, q-head, batch).  With xcd_remap the workgroups of
+// one (batch, kv-head) - which share K and V - are kept on one XCD (hardware
+// deals consecutive workgroup ids round-robin over the 8 XCDs), so K/V are
+// fetched from HBM once per XCD L2 instead of once per L2 of every XCD.
+// Row tiles are visited last-first: under a causal mask the last tiles are
+// the longest, and starting them first shortens the tail of the launch.
+FA2_DEV void decode_block(const KArgs& a, int& mt, int& h, int& b) {
+	int id = blockIdx.x;
+	int r = a.Hq / a.Hkv;
+	int per_group = a.mtiles * r;
+	int grp, within;
+	if (a.xcd_remap) {
+		int xcd = id & 7, j = id >> 3;
+		grp = (j / per_group) * 8 + xcd;
+		within = j % per_group;
+	} else {
+		grp = id / per_group;
+		within = id % per_group;
+	}
+	int hk = grp % a.Hkv;
+	b = grp / a.Hkv;
+	mt = a.mtiles - 1 - within / r;
+	h = hk * r + within % r;
+}
+
+// four consecutive bias values bias[row][col..col+3] as floats
+FA2_DEV f32x4 load_bias4(const char* rowp, int col, int dtype, bool vec_ok, int ncols) {
+	f32x4 out;
+	if (vec_ok && col + 3 < ncols) {
+		if (dtype == 3) {
+			out = *(const f32x4*)(rowp + (int64_t)col * 4);
+		} else if (dtype == 2) {
+			bf16x4 t = *(const bf16x4*)(rowp + (int64_t)col * 2);
+			out = __builtin_convertvector(t, f32x4);
+		} else {
+			f16x4 t = *(const f16x4*)(rowp + (int64_t)col * 2);
+			out = __builtin_convertvector(t, f32x4);
+		}
+	} else {
+#pragma unroll
+		for (int e = 0; e < 4; ++e) {
+			float x = 0.f;
+			if (col + e < ncols) {
+				if (dtype == 3)
+					x = *(const float*)(rowp + (int64_t)(col + e) * 4);
+				else if (dtype == 2)
+					x = (float)*(const __bf16*)(rowp + (int64_t)(col + e) * 2);
+				else
+					x = (float)*(const _Float16*)(rowp + (int64_t)(col + e) * 2);
+			}
+			out[e] = x;
+		}
+	}
+	return out;
+}
+
+template <typename T, int D, int NW, int QB, bool BIAS, bool DROP>
+__global__ __launch_bounds__(NW * 64) void fwd_kernel(const KArgs a) {
+	typedef typename T::V8 V8;
+	constexpr int BM = NW * QB * 32;
+	constexpr int BN = kFwdBN;
+	constexpr int KB = BN / 32;   // 32-key blocks per tile
+	constexpr int KS = D / 16;    // MFMA k-steps along D
+	constexpr int DB = D / 32;    // 32-wide blocks of the head dim
+	constexpr int NT = NW * 64;
+	constexpr int TILE_BYTES = BN * D * 2;
+
+	__shared__ __attribute__((aligned(1024))) char smem[4 * TILE_BYTES];
+	FA2_LDS char* lds = (FA2_LDS char*)smem;
+	// layout: K[0] K[1] V[0] V[1]
+
+	int mt, h, b;
+	decode_block(a, mt, h, b);
+	const int hk = h / (a.Hq / a.Hkv);
+	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+	const int g = lane >> 5, c = lane & 31;
+
+	int sq_eff = a.Sq, sk_eff = a.Sk;
+	if (a.seqlens) {
+		int len = a.seqlens[b];
+		len = len < 0 ? 0 : (len > a.Sk ? a.Sk : len);
+		sq_eff = len < a.Sq ? len : a.Sq;
+		sk_eff = len;
+	}
+	const int off = sk_eff - sq_eff;  // causal: key j allowed for row i iff j <= i + off
+	const int m0 = mt * BM;
+	const int wm0 = m0 + w * (QB * 32);
+
+	// keys this row tile can see
+	int kv_end = sk_eff;
+	if (a.causal) {
+		int last_row = (m0 + BM - 1 < sq_eff - 1) ? m0 + BM - 1 : sq_eff - 1;
+		int e = last_row + off + 1;
+		kv_end = e < kv_end ? e : kv_end;
+	}
+	if (m0 >= sq_eff) kv_end = 0;
+	const int ntiles = kv_end > 0 ? (kv_end + BN - 1) / BN : 0;
+
+	// per-lane last allowed key for each of this lane's rows
+	int jmax[QB];
+	int qrow[QB];
+#pragma unroll
+	for (int qb = 0; qb < QB; ++qb) {
+		int i = wm0 + 32 * qb + c;
+		qrow[qb] = i;
+		int jm = sk_eff - 1;
+		if (a.causal) jm = (i + off < jm) ? i + off : jm;
+		if (i >= sq_eff) jm = -1;
+		jmax[qb] = jm;
+	}
+	// wave-uniform bounds of jmax over the wave's rows
+	int wave_jmin, wave_jmax;
+	{
+		int first = wm0, last = wm0 + QB * 32 - 1;
+		if (first >= sq_eff) {
+			wave_jmin = wave_jmax = -1;
+		} else {
+			wave_jmax = sk_eff - 1;
+			wave_jmin = sk_eff - 1;
+			int lastv = last < sq_eff - 1 ? last : sq_eff - 1;
+			if (a.causal) {
+				wave_jmax = (lastv + off < wave_jmax) ? lastv + off : wave_jmax;
+				wave_jmin = (first + off < wave_jmin) ? first + off : wave_jmin;
+			}
+			if (last >= sq_eff) wave_jmin = -1;
+		}
+	}
+
+	const char* kbase = a.k.ptr + (int64_t)b * a.k.sb + (int64_t)hk * a.k.sh;
+	const char* vbase = a.v.ptr + (int64_t)b * a.v.sb + (int64_t)hk * a.v.sh;
+
+	// prologue: first K/V tile in flight while Q is fetched
+	if (ntiles > 0) {
+		int rows = sk_eff < BN ? sk_eff : BN;
+		tile_load_async<D, BN, NT>(lds, kbase, a.k.ss, rows, tid);
+		tile_load_async<D, BN, NT>(lds + 2 * TILE_BYTES, vbase, a.v.ss, rows, tid);
+	}
+
+	// Q fragments (B operand of S^T): lane holds Q[row c][16ks + 8g .. +7]
+	V8 qf[QB][KS];
+	{
+		const char* qbase = a.q.ptr + (int64_t)b * a.q.sb + (int64_t)h * a.q.sh;
+#pragma unroll
+		for (int qb = 0; qb < QB; ++qb) {
+			int i = qrow[qb] < a.Sq ? qrow[qb] : a.Sq - 1;
+			const char* rp = qbase + (int64_t)i * a.q.ss + g * 16;
+#pragma unroll
+			for (int ks = 0; ks < KS; ++ks) qf[qb][ks] = *(const V8*)(rp + ks * 32);
+		}
+	}
+
+	f32x16 oacc[QB][DB];
+	float mrow[QB], lrow[QB];
+#pragma unroll
+	for (int qb = 0; qb < QB; ++qb) {
+		mrow[qb] = -INFINITY;
+		lrow[qb] = 0.f;
+#pragma unroll
+		for (int db = 0; db < DB; ++db)
+#pragma unroll
+			for (int i = 0; i < 16; ++i) oacc[qb][db][i] = 0.f;
+	}
+
+	const float c1 = BIAS ? a.scale : a.scale * kLog2e;  // score -> softmax domain
+	const char* bias_base = nullptr;
+	if constexpr (BIAS) {
+		int hb = a.bias_group ? hk : h;
+		bias_base = a.bias + (int64_t)b * a.bias_sb + (int64_t)hb * a.bias_sh;
+	}
+
+	for (int t = 0; t < ntiles; ++t) {
+		const int n0 = t * BN;
+		const int buf = t & 1;
+		wait_async_loads();
+		__syncthreads();
+		if (t + 1 < ntiles) {
+			int n1 = n0 + BN;
+			int rows = sk_eff - n1 < BN ? sk_eff - n1 : BN;
+			tile_load_async<D, BN, NT>(lds + (buf ^ 1) * TILE_BYTES, kbase + (int64_t)n1 * a.k.ss, a.k.ss, rows, tid);
+			tile_load_async<D, BN, NT>(lds + (2 + (buf ^ 1)) * TILE_BYTES, vbase + (int64_t)n1 * a.v.ss, a.v.ss, rows, tid);
+		}
+		if (n0 > wave_jmax) continue;  // whole tile masked for this wave (uniform)
+		const bool need_mask = n0 + BN - 1 > wave_jmin;
+		const FA2_LDS char* kt = lds + buf * TILE_BYTES;
+		const FA2_LDS char* vt = lds + (2 + buf) * TILE_BYTES;
+
+		// bias tile, fetched ahead of the matrix products
+		f32x4 bv[BIAS ? KB : 1][BIAS ? QB : 1][4];
+		if constexpr (BIAS) {
+#pragma unroll
+			for (int qb = 0; qb < QB; ++qb) {
+				int i = qrow[qb] < a.Sq ? qrow[qb] : a.Sq - 1;
+				const char* rowp = bias_base + (int64_t)i * a.bias_sm;
+#pragma unroll
+				for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+					for (int aa = 0; aa < 4; ++aa)
+						bv[kb][qb][aa] = load_bias4(rowp, n0 + 32 * kb + 8 * aa + 4 * g, a.bias_dtype, a.bias_vec4, a.Sk);
+			}
+		}
+
+		// S^T = K Q^T
+		f32x16 s[KB][QB];
+#pragma unroll
+		for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+			for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+				for (int i = 0; i < 16; ++i) s[kb][qb][i] = 0.f;
+#pragma unroll
+		for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+			for (int kb = 0; kb < KB; ++kb) {
+				V8 kf = lds_frag<T, D>(kt, 32 * kb, ks, lane);
+#pragma unroll
+				for (int qb = 0; qb < QB; ++qb) s[kb][qb] = mfma32(kf, qf[qb][ks], s[kb][qb]);
+			}
+
+		// online softmax, one query row per lane
+		V8 pf[QB][BN / 16];
+#pragma unroll
+		for (int qb = 0; qb < QB; ++qb) {
+			float mx = -INFINITY;
+#pragma unroll
+			for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+				for (int i = 0; i < 16; ++i) {
+					float x;
+					if constexpr (BIAS)
+						x = __builtin_fmaf(s[kb][qb][i], c1, bv[kb][qb][i >> 2][i & 3]);
+					else
+						x = s[kb][qb][i] * c1;
+					if (need_mask) {
+						int j = n0 + 32 * kb + 8 * (i >> 2) + 4 * g + (i & 3);
+						x = j <= jmax[qb] ? x : -INFINITY;
+					}
+					s[kb][qb][i] = x;
+					mx = __builtin_fmaxf(mx, x);
+				}
+			mx = pair_max(mx);
+			float m_new = __builtin_fmaxf(mrow[qb], mx);
+			float m_use = m_new == -INFINITY ? 0.f : m_new;
+			float alpha = BIAS ? exp2_fast((mrow[qb] - m_use) * kLog2e) : exp2_fast(mrow[qb] - m_use);
+			mrow[qb] = m_new;
+			float lsum = 0.f;
+#pragma unroll
+			for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+				for (int i = 0; i < 16; ++i) {
+					float p = BIAS ? exp2_fast((s[kb][qb][i] - m_use) * kLog2e) : exp2_fast(s[kb][qb][i] - m_use);
+					lsum += p;
+					s[kb][qb][i] = p;
+				}
+			lrow[qb] = lrow[qb] * alpha + lsum;
+			if constexpr (DROP) {
+#pragma unroll
+				for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+					for (int aa = 0; aa < 4; ++aa) {
+						int j4 = (n0 + 32 * kb + 8 * aa + 4 * g) >> 2;
+						u32x4 rnd = philox4x32_10((uint32_t)j4, (uint32_t)qrow[qb], (uint32_t)h, (uint32_t)b, a.drop_k0, a.drop_k1);
+#pragma unroll
+						for (int e = 0; e < 4; ++e)
+							s[kb][qb][4 * aa + e] = rnd[e] >= a.drop_thr ? s[kb][qb][4 * aa + e] : 0.f;
+					}
+			}
+#pragma unroll
+			for (int db = 0; db < DB; ++db)
+#pragma unroll
+				for (int i = 0; i < 16; ++i) oacc[qb][db][i] *= alpha;
+#pragma unroll
+			for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+				for (int hf = 0; hf < 2; ++hf) {
+					const f32x16& r = s[kb][qb];
+					pf[qb][2 * kb + hf] = pack8<T>(r[8 * hf + 0], r[8 * hf + 1], r[8 * hf + 2], r[8 * hf + 3], r[8 * hf + 4],
+					                               r[8 * hf + 5], r[8 * hf + 6], r[8 * hf + 7]);
+				}
+		}
+
+		// O^T += V^T P^T
+#pragma unroll
+		for (int kk = 0; kk < BN / 16; ++kk)
+#pragma unroll
+			for (int db = 0; db < DB; ++db) {
+				V8 vf = lds_frag_tr<T, D>(vt, 16 * kk, 32 * db, lane);
+#pragma unroll
+				for (int qb = 0; qb < QB; ++qb) oacc[qb][db] = mfma32(vf, pf[qb][kk], oacc[qb][db]);
+			}
+	}
+
+	// epilogue: normalise, store O (lane: row c, four consecutive d per store) and LSE
+	char* obase = a.o.ptr + (int64_t)b * a.o.sb + (int64_t)h * a.o.sh;
+#pragma unroll
+	for (int qb = 0; qb < QB; ++qb) {
+		float lt = pair_sum(lrow[qb]);
+		float inv = lt > 0.f ? 1.f / lt : 0.f;
+		if constexpr (DROP) inv *= a.drop_inv_keep;
+		int i = qrow[qb];
+		if (i < a.Sq) {
+			char* rp = obase + (int64_t)i * a.o.ss;
+#pragma unroll
+			for (int db = 0; db < DB; ++db)
+#pragma unroll
+				for (int aa = 0; aa < 4; ++aa) {
+					const f32x16& r = oacc[qb][db];
+					u32x2 pk = {pack2<typename T::V2>(r[4 * aa] * inv, r[4 * aa + 1] * inv),
+					            pack2<typename T::V2>(r[4 * aa + 2] * inv, r[4 * aa + 3] * inv)};
+					*(u32x2*)(rp + (32 * db + 8 * aa + 4 * g) * 2) = pk;
+				}
+			if (g == 0) {
+				float lse;
+				if (lt > 0.f)
+					lse = BIAS ? mrow[qb] + log2_fast(lt) * kLn2 : (mrow[qb] + log2_fast(lt)) * kLn2;
+				else
+					lse = -INFINITY;
+				a.lse[((int64_t)b * a.Hq + h) * a.Sq + i] = lse;
+			}
+		}
+	}
+}
+
+template <typename T, int D>
+struct FwdCfg {
+	static constexpr int NW = 4;
+	static constexpr int QB = D <= 128 ? 2 : 1;
+	static constexpr int BM = NW * QB * 32;
+};
+
+template <typename T, int D>
+hipError_t launch_fwd_t(bool bias, bool drop, KArgs& a, hipStream_t s) {
+	typedef FwdCfg<T, D> C;
+	a.mtiles = (a.Sq + C::BM - 1) / C::BM;
+	int groups = a.B * a.Hkv;
+	a.xcd_remap = (groups % 8 == 0) ? 1 : 0;
+	dim3 grid((unsigned)(a.mtiles * a.B * a.Hq)), block(C::NW * 64);
+	if (bias && drop)
+		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, true, true>), grid, block, 0, s, a);
+	else if (bias)
+		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, true, false>), grid, block, 0, s, a);
+	else if (drop)
+		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, false, true>), grid, block, 0, s, a);
+	else
+		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, false, false>), grid, block, 0, s, a);
+	return hipGetLastError();
+}
+
+}  // namespace fa2

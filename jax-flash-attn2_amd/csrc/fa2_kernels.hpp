@@ -1,0 +1,56 @@
+// Host <-> kernel argument block and the launchers the C ABI dispatches to.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fa2 {
+
+// Everything a kernel needs, by value.  Strides are in BYTES here (the C ABI
+// takes element strides; the launcher converts).
+struct KTensor {
+	char* ptr;
+	int64_t sb, ss, sh;
+};
+
+struct KArgs {
+	KTensor q, k, v, o, dout, dq, dk, dv;
+	float* lse;      // [B, Hq, Sq] natural-log logsumexp
+	float* delta;    // [B, Hq, Sq] rowsum(dO * O)  (backward scratch)
+	const char* bias;
+	int64_t bias_sb, bias_sh, bias_sm;  // bytes
+	int bias_dtype;  // FA2_FP16 / FA2_BF16 / FA2_FP32
+	int bias_group;  // head axis of bias indexed by kv-head
+	int bias_vec4;   // rows are 4-element aligned: vector loads allowed
+	const int32_t* seqlens;
+	int B, Sq, Sk, Hq, Hkv;
+	int causal;
+	float scale;
+	uint32_t drop_k0, drop_k1, drop_thr;
+	float drop_inv_keep;
+	int mtiles;      // number of row tiles of the launched kernel
+	int xcd_remap;   // 1: group-major placement of workgroups on the 8 XCDs
+};
+
+// dtype: FA2_FP16 / FA2_BF16.  Return hipError_t of the launch.
+hipError_t launch_fwd(int dtype, int D, bool bias, bool drop, KArgs& a, hipStream_t s);
+hipError_t launch_bwd(int dtype, int D, bool bias, bool drop, KArgs& a, hipStream_t s);
+hipError_t launch_dropout_mask(uint8_t* keep, int B, int H, int Sq, int Sk, uint32_t k0, uint32_t k1, uint32_t thr,
+                               hipStream_t s);
+
+// Per-(dtype, D) translation units provide these.
+#define FA2_DECL_FWD(TAG, DD) hipError_t launch_fwd_##TAG##_##DD(bool bias, bool drop, KArgs& a, hipStream_t s);
+#define FA2_DECL_BWD(TAG, DD) hipError_t launch_bwd_##TAG##_##DD(bool bias, bool drop, KArgs& a, hipStream_t s);
+FA2_DECL_FWD(bf16, 64)
+FA2_DECL_FWD(bf16, 128)
+FA2_DECL_FWD(bf16, 256)
+FA2_DECL_FWD(fp16, 64)
+FA2_DECL_FWD(fp16, 128)
+FA2_DECL_FWD(fp16, 256)
+FA2_DECL_BWD(bf16, 64)
+FA2_DECL_BWD(bf16, 128)
+FA2_DECL_BWD(bf16, 256)
+FA2_DECL_BWD(fp16, 64)
+FA2_DECL_BWD(fp16, 128)
+FA2_DECL_BWD(fp16, 256)
+
+}  // namespace fa2

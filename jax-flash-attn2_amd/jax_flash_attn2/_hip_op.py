@@ -1,0 +1,226 @@
+"""The HIP attention operator: forward / backward calls into libfa2_hip.so and
+the differentiation rule that ties them together.
+
+Takes the place of the reference's per-platform operator
+`jax_flash_attn2/flash_attention_triton/_flash_attention.py:27-157`
+(`_jax_fwd_attention_call`, `_jax_bwd_attention_call`, `flash_attention_call`,
+`flash_attention`): same argument list, same residuals (q, k, v, bias, mask,
+out, lse, seed), gradients for q, k, v only.
+
+Arrays here are torch tensors on a ROCm device - torch is used for device
+memory and the stream handle only; every number is produced by the C ABI.  The
+same two entry points are what the XLA-FFI handlers in csrc/fa2_xla_ffi.cc
+forward to when the caller is JAX.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import math
+import typing as tp
+
+import torch
+
+from . import _lib
+from ._lib import FA2_BF16, FA2_FP16, FA2_FP32, Fa2Tensor
+
+_DTYPES = {torch.float16: FA2_FP16, torch.bfloat16: FA2_BF16}
+_BIAS_DTYPES = {torch.float16: FA2_FP16, torch.bfloat16: FA2_BF16, torch.float32: FA2_FP32}
+
+
+def _stream_ptr(device) -> int:
+	return torch.cuda.current_stream(device).cuda_stream
+
+
+def _t4(x: torch.Tensor) -> Fa2Tensor:
+	"""[B, S, H, D] tensor -> pointer + element strides (D stride must be 1)."""
+	t = Fa2Tensor()
+	t.ptr = x.data_ptr()
+	t.stride_b, t.stride_s, t.stride_h = x.stride(0), x.stride(1), x.stride(2)
+	return t
+
+
+def _usable(x: torch.Tensor) -> torch.Tensor:
+	"""Kernels read 16 bytes at a time along D: unit D stride, 16-byte aligned rows."""
+	if x.stride(3) != 1 or any(s % 8 for s in x.stride()[:3]) or x.data_ptr() % 16:
+		return x.contiguous()
+	return x
+
+
+def check_shapes(q, k, v, bias, attention_mask):
+	"""Validation of `_fwd_attention_kernel_call` (_forward_triton.py:474-495) and
+	`calc_bias_strides` (_utils.py:151-193), with the reference's messages."""
+	batch, QSeq, nheads_q, head_dim = q.shape
+	_, KSeq, nheads_kv, _ = k.shape
+	expected_kv_shape = (batch, KSeq, nheads_kv, head_dim)
+	if attention_mask is not None:
+		assert bias is None, "Attention mask is not supported along with attention bias. Just use bias instead."
+		assert QSeq == KSeq, "Attention mask is not supported with QSeq != KSeq"
+	assert tuple(k.shape) == expected_kv_shape, (
+		f"key shape is k.shape = {tuple(k.shape)} and we excepted it to be like expected_kv_shape = {expected_kv_shape}"
+	)
+	assert tuple(v.shape) == expected_kv_shape, (
+		f"value shape is v.shape = {tuple(v.shape)} and we excepted it to be like expected_kv_shape = {expected_kv_shape}"
+	)
+	assert nheads_q % nheads_kv == 0, f"nheads_q = {nheads_q} is not divisible by nheads_kv ={nheads_kv}"
+	assert q.dtype == k.dtype == v.dtype, "All tensors must have the same type"
+	assert q.dtype in _DTYPES, "Only support fp16 and bf16"
+	if bias is not None:
+		if bias.shape[2] != QSeq or bias.shape[3] != KSeq:
+			raise ValueError(
+				f"Bias tensor has incompatible sequence dimensions. "
+				f"Expected shape [..., {QSeq}, {KSeq}], but got [..., {bias.shape[2]}, {bias.shape[3]}]. "
+				f"Full bias shape: {tuple(bias.shape)}"
+			)
+		if bias.shape[0] not in (1, batch):
+			raise ValueError(
+				f"Batch dimension mismatch in bias tensor. "
+				f"Expected either 1 (for broadcasting) or {batch} (batch size), "
+				f"but got {bias.shape[0]}. Consider reshaping your bias tensor."
+			)
+		if bias.shape[1] not in (1, nheads_q) and not (bias.shape[1] == nheads_kv):
+			raise ValueError(
+				f"Head dimension mismatch in bias tensor. "
+				f"Expected either 1 (for broadcasting) or {nheads_q} (number of heads), "
+				f"but got {bias.shape[1]}. Check that your bias tensor matches the model configuration."
+			)
+
+
+def _fill_common(p, q, k, v, bias, seqlens, scale, p_drop, causal, seed):
+	B, Sq, Hq, D = q.shape
+	Sk, Hkv = k.shape[1], k.shape[2]
+	p.dtype = _DTYPES[q.dtype]
+	p.B, p.Sq, p.Sk, p.Hq, p.Hkv, p.D = B, Sq, Sk, Hq, Hkv, D
+	p.causal = 1 if causal else 0
+	p.scale = float(scale)
+	p.p_drop = float(p_drop)
+	p.seed = int(seed) & 0xFFFFFFFFFFFFFFFF
+	p.q, p.k, p.v = _t4(q), _t4(k), _t4(v)
+	if bias is not None:
+		p.bias = bias.data_ptr()
+		p.bias_dtype = _BIAS_DTYPES[bias.dtype]
+		# broadcast rules of calc_bias_strides (_utils.py:169-190): size-1 axes get stride 0.
+		p.bias_stride_b = 0 if bias.shape[0] == 1 else bias.stride(0)
+		p.bias_stride_h = 0 if bias.shape[1] == 1 else bias.stride(1)
+		p.bias_stride_m = bias.stride(2)
+		# a bias with Hkv heads is read per KV group instead of being repeated to Hq heads
+		# (the facade materialises that repeat, flash_attention.py:161-164)
+		p.bias_group = 1 if (bias.shape[1] == Hkv and Hkv != Hq and bias.shape[1] != 1) else 0
+	if seqlens is not None:
+		p.seqlens = seqlens.data_ptr()
+
+
+def _prep_bias(bias):
+	if bias is None:
+		return None
+	if bias.dtype not in _BIAS_DTYPES:
+		bias = bias.to(torch.float32)
+	if bias.stride(3) != 1:
+		bias = bias.contiguous()
+	return bias
+
+
+def _seqlens_from_mask(attention_mask, q):
+	"""The reference's GPU path takes a right-padded 2-D validity mask [B, S] and
+	packs the valid tokens (_forward_triton.py:499-510).  Here the mask is reduced
+	to one length per batch row which the kernels consume directly."""
+	if attention_mask is None:
+		return None
+	if attention_mask.dim() != 2:
+		raise ValueError("attention_mask must be a 2-D [batch, seq] right-padded validity mask; use bias for general masks")
+	return attention_mask.to(device=q.device).ne(0).sum(dim=1, dtype=torch.int32).contiguous()
+
+
+def fwd(q, k, v, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, causal=False, dropout_seed=None):
+	"""Returns (out [B,Sq,Hq,D] in q.dtype, lse [B,Hq,Sq] fp32 natural log)."""
+	lib = _lib.load()
+	q, k, v = _usable(q), _usable(k), _usable(v)
+	bias = _prep_bias(bias)
+	B, Sq, Hq, D = q.shape
+	scale = 1.0 / math.sqrt(D) if softmax_scale is None else softmax_scale
+	out = torch.empty((B, Sq, Hq, D), dtype=q.dtype, device=q.device)
+	lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
+	p = _lib.new_params()
+	_fill_common(p, q, k, v, bias, seqlens, scale, dropout_prob, causal, dropout_seed or 0)
+	p.o = _t4(out)
+	p.lse = lse.data_ptr()
+	_lib.check(lib.fa2_fwd(ctypes.byref(p), _stream_ptr(q.device)))
+	return out, lse
+
+
+def bwd(q, k, v, out, lse, dout, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, causal=False,
+        dropout_seed=None):
+	"""Returns (dq, dk, dv) in the dtypes of q, k, v; dk/dv summed over each KV group."""
+	lib = _lib.load()
+	q, k, v, out, dout = _usable(q), _usable(k), _usable(v), _usable(out), _usable(dout)
+	bias = _prep_bias(bias)
+	B, Sq, Hq, D = q.shape
+	scale = 1.0 / math.sqrt(D) if softmax_scale is None else softmax_scale
+	dq = torch.empty_like(q, memory_format=torch.contiguous_format)
+	dk = torch.empty_like(k, memory_format=torch.contiguous_format)
+	dv = torch.empty_like(v, memory_format=torch.contiguous_format)
+	p = _lib.new_params()
+	_fill_common(p, q, k, v, bias, seqlens, scale, dropout_prob, causal, dropout_seed or 0)
+	p.o = _t4(out)
+	p.lse = lse.data_ptr()
+	p.dout, p.dq, p.dk, p.dv = _t4(dout), _t4(dq), _t4(dk), _t4(dv)
+	need = lib.fa2_bwd_scratch_bytes(ctypes.byref(p))
+	scratch = torch.empty((max(need, 256),), dtype=torch.uint8, device=q.device)
+	p.scratch = scratch.data_ptr()
+	p.scratch_bytes = scratch.numel()
+	_lib.check(lib.fa2_bwd(ctypes.byref(p), _stream_ptr(q.device)))
+	return dq, dk, dv
+
+
+def dropout_mask(B, H, Sq, Sk, dropout_prob, dropout_seed, device) -> torch.Tensor:
+	"""keep[b,h,i,j] (uint8) exactly as the kernels regenerate it."""
+	lib = _lib.load()
+	keep = torch.empty((B, H, Sq, Sk), dtype=torch.uint8, device=device)
+	p = _lib.new_params()
+	p.B, p.Hq, p.Hkv, p.Sq, p.Sk, p.D = B, H, H, Sq, Sk, 64
+	p.p_drop = float(dropout_prob)
+	p.seed = int(dropout_seed or 0) & 0xFFFFFFFFFFFFFFFF
+	_lib.check(lib.fa2_dropout_mask(ctypes.byref(p), keep.data_ptr(), _stream_ptr(device)))
+	return keep
+
+
+class _FlashAttentionFn(torch.autograd.Function):
+	"""Differentiation rule; the torch spelling of the reference's
+	`flash_attention_call.defvjp(_jax_fwd_attention_call, _jax_bwd_attention_call)`
+	(_flash_attention.py:119-122).  Returns (dq, dk, dv) and None for everything else."""
+
+	@staticmethod
+	def forward(ctx, q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed):
+		out, lse = fwd(q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed)
+		ctx.save_for_backward(q, k, v, bias, seqlens, out, lse)
+		ctx.cfg = (softmax_scale, dropout_prob, causal, dropout_seed)
+		return out
+
+	@staticmethod
+	def backward(ctx, dout):
+		q, k, v, bias, seqlens, out, lse = ctx.saved_tensors
+		softmax_scale, dropout_prob, causal, dropout_seed = ctx.cfg
+		dq, dk, dv = bwd(q, k, v, out, lse, dout, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed)
+		return dq, dk, dv, None, None, None, None, None, None
+
+
+def flash_attention(
+	q,
+	k,
+	v,
+	attention_mask=None,
+	bias=None,
+	softmax_scale: tp.Optional[float] = None,
+	dropout_prob: float = 0.0,
+	causal: bool = False,
+	dropout_seed: tp.Optional[int] = None,
+	varlen_mode: bool = True,
+):
+	"""Same signature as the reference's `triton_flash_attention`
+	(_flash_attention.py:125-157).  `varlen_mode` is accepted for source
+	compatibility; padded batches are always handled in-kernel from per-row
+	lengths, never by packing."""
+	del varlen_mode
+	check_shapes(q, k, v, bias, attention_mask)
+	seqlens = _seqlens_from_mask(attention_mask, q)
+	return _FlashAttentionFn.apply(q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed)
