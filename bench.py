@@ -1,0 +1,220 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+A step = one forward + one backward call through the C ABI (fa2_fwd, fa2_bwd)
+on inputs already resident in HBM.  Default workload: the Llama-3-8B-style
+prefill shape (B=4, S=4096, Hq=32, Hkv=8, D=128, bf16, causal).
+
+Prints ONE JSON line: whole-step throughput in TFLOP/s (FlashAttention-2 FLOP
+convention: fwd = 4*B*Hq*Sq*Sk*D, halved when causal; bwd = 2.5 x fwd), the
+roofline entry of the dominant kernel (timed live with HIP events on the
+launch stream) and a CPU baseline (the NumPy restatement of the reference's
+JAX-platform blockwise algorithm on a bounded sample).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "jax-flash-attn2_amd"))
+
+PEAK_TFLOPS = {"bf16": 2516.6, "fp16": 2516.6}  # dense MFMA, 256 CU x 2.4 GHz x 4096 FLOP/clk/CU
+HBM_PEAK_GBS = 8000.0
+
+WORKLOADS = {
+	# name: B, Sq, Sk, Hq, Hkv, D, dtype, causal, bias, dropout, backward
+	"c1": dict(B=2, S=512, Hq=16, Hkv=4, D=64, dtype="fp16", causal=True, bias=False, p=0.0, bwd=False,
+	           desc="README shape B2 Hq16 Hkv4 S512 D64 fp16 causal, forward only"),
+	"c2": dict(B=4, S=4096, Hq=32, Hkv=8, D=128, dtype="bf16", causal=True, bias=False, p=0.0, bwd=True,
+	           desc="Llama-3-8B prefill B4 S4096 Hq32 Hkv8 D128 bf16 causal, forward+backward"),
+	"c3": dict(B=8, S=2048, Hq=16, Hkv=16, D=64, dtype="bf16", causal=False, bias=True, p=0.0, bwd=True,
+	           desc="padded MHA B8 S2048 H16 D64 bf16, bias [B,1,S,S] with mask folded in, forward+backward"),
+	"c4": dict(B=1, S=32768, Hq=64, Hkv=8, D=128, dtype="bf16", causal=True, bias=False, p=0.0, bwd=True,
+	           desc="long context B1 S32768 Hq64 Hkv8 D128 bf16 causal, forward+backward"),
+	"c5": dict(B=8, S=2048, Hq=16, Hkv=16, D=256, dtype="bf16", causal=True, bias=False, p=0.1, bwd=True,
+	           desc="dropout, wide heads B8 S2048 H16 D256 bf16 causal p=0.1 seed=42, forward+backward"),
+}
+
+
+def fwd_flops(w):
+	f = 4.0 * w["B"] * w["Hq"] * w["S"] * w["S"] * w["D"]
+	return f / 2 if w["causal"] else f
+
+
+def make_inputs(w, device):
+	import torch
+
+	dt = torch.bfloat16 if w["dtype"] == "bf16" else torch.float16
+	g = torch.Generator(device=device)
+	B, S, Hq, Hkv, D = w["B"], w["S"], w["Hq"], w["Hkv"], w["D"]
+	mul = 1.0 if w is WORKLOADS["c1"] else 0.5
+
+	def rnd(seed, shape, m):
+		g.manual_seed(seed)
+		return (torch.randn(shape, generator=g, device=device, dtype=torch.float32) * m).to(dt)
+
+	q = rnd(0, (B, S, Hq, D), mul)
+	k = rnd(1, (B, S, Hkv, D), mul)
+	v = rnd(2, (B, S, Hkv, D), mul)
+	do = rnd(3, (B, S, Hq, D), 1.0)
+	bias = None
+	if w["bias"]:
+		# bias[b,0,i,j] = 1/(1+|i-j|) ; keys beyond a per-row valid length get finfo.min
+		i = torch.arange(S, device=device)
+		base = 1.0 / (1.0 + (i[:, None] - i[None, :]).abs().float())
+		g.manual_seed(4)
+		lens = torch.randint(S // 2, S + 1, (B,), generator=g, device=device)
+		valid = i[None, :] < lens[:, None]
+		bias = base[None, None].expand(B, 1, S, S).clone()
+		bias = torch.where(valid[:, None, None, :], bias, torch.full_like(bias, torch.finfo(dt).min)).to(dt)
+	return q, k, v, do, bias
+
+
+def event_time_ms(fn, iters, torch):
+	"""Average duration of fn() over `iters` launches, HIP events on the current stream."""
+	start = torch.cuda.Event(enable_timing=True)
+	stop = torch.cuda.Event(enable_timing=True)
+	start.record()
+	for _ in range(iters):
+		fn()
+	stop.record()
+	stop.synchronize()
+	return start.elapsed_time(stop) / iters
+
+
+def cpu_baseline(w):
+	"""Reference JAX-platform algorithm (NumPy restatement) on a bounded sample of the workload."""
+	sys.path.insert(0, os.path.join(ROOT, "oracle"))
+	import numpy as np
+
+	import fa2_oracle as O
+
+	r = w["Hq"] // w["Hkv"]
+	B, S, D = 1, min(w["S"], 4096), w["D"]
+	Hkv = min(2, w["Hkv"])
+	Hq = Hkv * r
+	rng = np.random.default_rng(0)
+	q = rng.standard_normal((B, S, Hq, D), dtype=np.float32) * 0.5
+	k = rng.standard_normal((B, S, Hkv, D), dtype=np.float32) * 0.5
+	v = rng.standard_normal((B, S, Hkv, D), dtype=np.float32) * 0.5
+	do = rng.standard_normal((B, S, Hq, D), dtype=np.float32)
+	t0 = time.perf_counter()
+	if w["bwd"]:
+		O.jax_platform_call(q, k, v, with_grads_for=do)
+	else:
+		O.jax_platform_call(q, k, v)
+	dt = time.perf_counter() - t0
+	# that branch of the reference never applies the causal mask: it computes the full S x S problem
+	flops = 4.0 * B * Hq * S * S * D * (3.5 if w["bwd"] else 1.0)
+	return {
+		"value": flops / dt / 1e12,
+		"unit": "TFLOP/s",
+		"cores": os.cpu_count() if not os.environ.get("OMP_NUM_THREADS") else int(os.environ["OMP_NUM_THREADS"]),
+		"kind": "port",
+		"sample": f"B={B} Hq={Hq} Hkv={Hkv} S={S} D={D} fp32 non-causal (the reference's JAX branch ignores causal), "
+		          f"{'fwd+bwd' if w['bwd'] else 'fwd'}, blocks 128x128, {dt:.1f} s",
+		"seconds": dt,
+	}
+
+
+def main():
+	ap = argparse.ArgumentParser()
+	ap.add_argument("--gpus", type=int, default=1)
+	ap.add_argument("--steps", type=int, default=20)
+	ap.add_argument("--warmup", type=int, default=3)
+	ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+	ap.add_argument("--no-cpu-baseline", action="store_true")
+	args = ap.parse_args()
+	if args.gpus != 1:
+		print("bench.py: this build measures ONE GPU; --gpus N with N > 1 is not supported "
+		      "(attention shards over batch and KV-head groups without communication).", file=sys.stderr)
+		sys.exit(2)
+
+	import torch
+
+	from jax_flash_attn2 import _hip_op as op
+
+	if not torch.cuda.is_available():
+		print("bench.py: no GPU visible", file=sys.stderr)
+		sys.exit(1)
+	dev = torch.device("cuda:0")
+	w = WORKLOADS[args.workload]
+	q, k, v, do, bias = make_inputs(w, dev)
+	plan = op.Plan(q, k, v, dout=do if w["bwd"] else None, bias=bias, causal=w["causal"], dropout_prob=w["p"],
+	               dropout_seed=42 if w["p"] > 0 else None)
+
+	def step():
+		plan.forward()
+		if w["bwd"]:
+			plan.backward()
+
+	for _ in range(args.warmup):
+		step()
+	torch.cuda.synchronize()
+	t0 = time.perf_counter()
+	for _ in range(args.steps):
+		step()
+	torch.cuda.synchronize()
+	ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
+	ff = fwd_flops(w)
+	total = ff * (3.5 if w["bwd"] else 1.0)
+	tflops = total / (ms * 1e-3) / 1e12
+
+	# per-kernel durations, HIP events on the launch stream
+	it = max(3, min(args.steps, 20))
+	kern = {"fwd": event_time_ms(plan.forward, it, torch)}
+	alg = {"fwd": ff}
+	if w["bwd"]:
+		kern["bwd_delta"] = event_time_ms(lambda: plan.backward(1), it, torch)
+		kern["bwd_dkdv"] = event_time_ms(lambda: plan.backward(2), it, torch)
+		kern["bwd_dq"] = event_time_ms(lambda: plan.backward(4), it, torch)
+		# 5-product convention: S, dP, dV, dK belong to the dK/dV kernel (4 x 0.5 fwd), dQ to the dQ kernel;
+		# the dQ kernel's recomputation of S and dP is not counted.
+		alg["bwd_dkdv"] = 2.0 * ff
+		alg["bwd_dq"] = 0.5 * ff
+	dom = max((n for n in kern if n in alg), key=lambda n: kern[n])
+	peak = PEAK_TFLOPS[w["dtype"]]
+	achieved = alg[dom] / (kern[dom] * 1e-3) / 1e12
+	roofline = {
+		"kernel": dom,
+		"bound": "mfma",
+		"achieved": achieved,
+		"peak": peak,
+		"unit": "TFLOP/s",
+		"frac": achieved / peak,
+		"traffic": None,
+		"kernel_ms": {n: round(t, 4) for n, t in kern.items()},
+		"kernel_tflops": {n: round(alg[n] / (kern[n] * 1e-3) / 1e12, 1) for n in kern if n in alg},
+	}
+
+	out = {
+		"metric": "attention TFLOP/s fwd+bwd (bf16 causal)" if args.workload == "c2" else f"attention TFLOP/s ({args.workload})",
+		"value": tflops,
+		"unit": "TFLOP/s",
+		"n_gpus": 1,
+		"steps": args.steps,
+		"warmup": args.warmup,
+		"ms_per_step": ms,
+		"higher_is_better": True,
+		"scaling": "weak",
+		"vs_baseline": None,
+		"dtype": w["dtype"],
+		"data": "synthetic",
+		"config": {"workload": w["desc"]},
+		"pct_of_mfma_peak": 100.0 * tflops / peak,
+		"roofline": roofline,
+	}
+	if not args.no_cpu_baseline:
+		out["cpu_baseline"] = cpu_baseline(w)
+	print(json.dumps(out))
+
+
+if __name__ == "__main__":
+	main()

@@ -103,6 +103,13 @@ int fa2_fwd(const fa2_params* p, void* hip_stream);
  * (_backward_triton.py:1049-1161). */
 int fa2_bwd(const fa2_params* p, void* hip_stream);
 
+/* fa2_bwd restricted to some of its kernels, for per-kernel timing:
+ * bit 0 = delta pre-pass (`_attn_bwd_preprocess`, _backward_triton.py:79-147),
+ * bit 1 = dK/dV kernel (`_attn_bwd_block_dkdv`, :257-435),
+ * bit 2 = dQ kernel (`_attn_bwd_block_dq`, :519-709).  fa2_bwd == stages 7.
+ * The dK/dV and dQ kernels read the delta the pre-pass left in scratch. */
+int fa2_bwd_stages(const fa2_params* p, void* hip_stream, int stages);
+
 /* Bytes of scratch fa2_bwd needs for these dimensions (0 on invalid params). */
 size_t fa2_bwd_scratch_bytes(const fa2_params* p);
 

@@ -156,11 +156,14 @@ int fa2_fwd(const fa2_params* p, void* hip_stream) {
 	return e == hipSuccess ? FA2_OK : FA2_EHIP;
 }
 
-int fa2_bwd(const fa2_params* p, void* hip_stream) {
+int fa2_bwd(const fa2_params* p, void* hip_stream) { return fa2_bwd_stages(p, hip_stream, 7); }
+
+int fa2_bwd_stages(const fa2_params* p, void* hip_stream, int stages) {
 	int rc = validate(p, 1);
 	if (rc) return rc;
 	KArgs a;
 	fill(p, a);
+	a.stages = stages & 7;
 	a.dout = conv(p->dout);
 	a.dq = conv(p->dq);
 	a.dk = conv(p->dk);

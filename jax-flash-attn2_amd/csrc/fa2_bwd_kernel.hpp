@@ -555,17 +555,17 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 	typedef BwdCfg<T, D> C;
 	int groups = a.B * a.Hkv;
 	a.xcd_remap = (groups % 8 == 0) ? 1 : 0;
-	{
+	if (a.stages & 1) {
 		int64_t nrows = (int64_t)a.B * a.Sq * a.Hq;
 		constexpr int RPB = 256 / (D / 8);
 		hipLaunchKernelGGL((bwd_delta_kernel<T, D>), dim3((unsigned)((nrows + RPB - 1) / RPB)), dim3(256), 0, s, a);
 	}
-	{
+	if (a.stages & 2) {
 		a.mtiles = (a.Sk + C::KV_BN - 1) / C::KV_BN;
 		dim3 grid((unsigned)(a.mtiles * a.B * a.Hkv)), block(C::KV_NW * 64);
 		hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, C::KV_NW, C::KV_QB, BIAS, DROP>), grid, block, 0, s, a);
 	}
-	{
+	if (a.stages & 4) {
 		a.mtiles = (a.Sq + C::DQ_BM - 1) / C::DQ_BM;
 		dim3 grid((unsigned)(a.mtiles * a.B * a.Hq)), block(C::DQ_NW * 64);
 		hipLaunchKernelGGL((bwd_dq_kernel<T, D, C::DQ_NW, C::DQ_QB, BIAS, DROP>), grid, block, 0, s, a);

@@ -184,6 +184,46 @@ def dropout_mask(B, H, Sq, Sk, dropout_prob, dropout_seed, device) -> torch.Tens
 	return keep
 
 
+class Plan:
+	"""A filled parameter block with its output buffers, for callers that repeat
+	the same call (benchmarks, graph capture): `forward()` / `backward()` only
+	enqueue kernels, nothing is allocated per call."""
+
+	def __init__(self, q, k, v, dout=None, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, causal=False,
+	             dropout_seed=None):
+		self.lib = _lib.load()
+		self.q, self.k, self.v = _usable(q), _usable(k), _usable(v)
+		self.bias = _prep_bias(bias)
+		self.seqlens = seqlens
+		B, Sq, Hq, D = q.shape
+		scale = 1.0 / math.sqrt(D) if softmax_scale is None else softmax_scale
+		self.out = torch.empty((B, Sq, Hq, D), dtype=q.dtype, device=q.device)
+		self.lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
+		p = self.params = _lib.new_params()
+		_fill_common(p, self.q, self.k, self.v, self.bias, seqlens, scale, dropout_prob, causal, dropout_seed or 0)
+		p.o = _t4(self.out)
+		p.lse = self.lse.data_ptr()
+		self.device = q.device
+		if dout is not None:
+			self.dout = _usable(dout)
+			self.dq = torch.empty_like(self.q, memory_format=torch.contiguous_format)
+			self.dk = torch.empty_like(self.k, memory_format=torch.contiguous_format)
+			self.dv = torch.empty_like(self.v, memory_format=torch.contiguous_format)
+			p.dout, p.dq, p.dk, p.dv = _t4(self.dout), _t4(self.dq), _t4(self.dk), _t4(self.dv)
+			need = self.lib.fa2_bwd_scratch_bytes(ctypes.byref(p))
+			self.scratch = torch.empty((max(need, 256),), dtype=torch.uint8, device=q.device)
+			p.scratch = self.scratch.data_ptr()
+			p.scratch_bytes = self.scratch.numel()
+
+	def forward(self):
+		_lib.check(self.lib.fa2_fwd(ctypes.byref(self.params), _stream_ptr(self.device)))
+		return self.out, self.lse
+
+	def backward(self, stages: int = 7):
+		_lib.check(self.lib.fa2_bwd_stages(ctypes.byref(self.params), _stream_ptr(self.device), stages))
+		return self.dq, self.dk, self.dv
+
+
 class _FlashAttentionFn(torch.autograd.Function):
 	"""Differentiation rule; the torch spelling of the reference's
 	`flash_attention_call.defvjp(_jax_fwd_attention_call, _jax_bwd_attention_call)`

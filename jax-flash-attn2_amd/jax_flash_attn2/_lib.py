@@ -63,6 +63,7 @@ class Fa2Params(ctypes.Structure):
 EXPORTS = (
 	"fa2_fwd",
 	"fa2_bwd",
+	"fa2_bwd_stages",
 	"fa2_bwd_scratch_bytes",
 	"fa2_dropout_mask",
 	"fa2_validate",
@@ -99,6 +100,8 @@ def load() -> ctypes.CDLL:
 		lib.fa2_fwd.restype = ctypes.c_int
 		lib.fa2_bwd.argtypes = [pp, ctypes.c_void_p]
 		lib.fa2_bwd.restype = ctypes.c_int
+		lib.fa2_bwd_stages.argtypes = [pp, ctypes.c_void_p, ctypes.c_int]
+		lib.fa2_bwd_stages.restype = ctypes.c_int
 		lib.fa2_bwd_scratch_bytes.argtypes = [pp]
 		lib.fa2_bwd_scratch_bytes.restype = ctypes.c_size_t
 		lib.fa2_dropout_mask.argtypes = [pp, ctypes.c_void_p, ctypes.c_void_p]

@@ -76,8 +76,9 @@ def dropout_threshold(p_drop: float) -> int:
 	return min(int(math.floor(float(np.float32(p_drop)) * 4294967296.0)), 0xFFFFFFFF)
 
 
-def dropout_keep_mask(seed: int, p_drop: float, B: int, H: int, Sq: int, Sk: int) -> np.ndarray:
-	"""keep[b,h,i,j] (bool).
+def dropout_keep_mask(seed: int, p_drop: float, B: int, H: int, Sq: int, Sk: int, pos_offset=(0, 0, 0)) -> np.ndarray:
+	"""keep[b,h,i,j] (bool).  `pos_offset` = (b0, h0, i0) shifts the batch / head /
+	row indices, for checking a slice of a larger problem.
 
 	Counter = (j >> 2, i, h, b), key = (seed & 0xffffffff, seed >> 32); element
 	(i, j) uses output word j & 3 and is kept iff word >= floor(p * 2**32).
@@ -90,9 +91,10 @@ def dropout_keep_mask(seed: int, p_drop: float, B: int, H: int, Sq: int, Sk: int
 	k1 = (seed >> 32) & 0xFFFFFFFF
 	nj4 = (Sk + 3) // 4
 	j4 = np.arange(nj4, dtype=np.uint32)[None, None, None, :]
-	i = np.arange(Sq, dtype=np.uint32)[None, None, :, None]
-	h = np.arange(H, dtype=np.uint32)[None, :, None, None]
-	b = np.arange(B, dtype=np.uint32)[:, None, None, None]
+	b0, h0, i0 = pos_offset
+	i = (np.arange(Sq, dtype=np.uint32) + np.uint32(i0))[None, None, :, None]
+	h = (np.arange(H, dtype=np.uint32) + np.uint32(h0))[None, :, None, None]
+	b = (np.arange(B, dtype=np.uint32) + np.uint32(b0))[:, None, None, None]
 	w = philox4x32_10(j4, i, h, b, k0, k1)
 	words = np.stack(w, axis=-1).reshape(B, H, Sq, nj4 * 4)[..., :Sk]
 	return words >= thr
@@ -143,6 +145,26 @@ def allowed_mask(B, Sq, Sk, causal, seqlens=None):
 	return ok
 
 
+def _bh(x):
+	"""[B,S,H,D] -> contiguous [B,H,S,D] (BLAS-friendly)."""
+	return np.ascontiguousarray(np.swapaxes(x, 1, 2))
+
+
+def _qk(a, b):
+	"""einsum('bihd,bjhd->bhij') through batched matmul."""
+	return np.matmul(_bh(a), np.swapaxes(_bh(b), 2, 3))
+
+
+def _pv(p, v):
+	"""einsum('bhij,bjhd->bihd')."""
+	return np.swapaxes(np.matmul(p, _bh(v)), 1, 2)
+
+
+def _ptx(p, x):
+	"""einsum('bhij,bihd->bjhd')."""
+	return np.swapaxes(np.matmul(np.swapaxes(p, 2, 3), _bh(x)), 1, 2)
+
+
 def _scores(q, k, bias, scale, causal, seqlens, dtype):
 	B, Sq, Hq, D = q.shape
 	_, Sk, Hkv, _ = k.shape
@@ -151,7 +173,7 @@ def _scores(q, k, bias, scale, causal, seqlens, dtype):
 	r = Hq // Hkv
 	qf = np.asarray(q, dtype=dtype)
 	kf = np.repeat(np.asarray(k, dtype=dtype), r, axis=2)  # q-head h uses kv-head h // r
-	s = np.einsum("bihd,bjhd->bhij", qf, kf) * dtype(scale)
+	s = _qk(qf, kf) * dtype(scale)
 	bb = _expand_bias(bias, B, Hq, Hkv, Sq, Sk, dtype)
 	if bb is not None:
 		s = s + bb
@@ -161,7 +183,7 @@ def _scores(q, k, bias, scale, causal, seqlens, dtype):
 
 
 def attention_fwd(q, k, v, bias=None, causal=False, scale=None, seqlens=None,
-                  p_drop=0.0, seed=0, dtype=np.float64, return_probs=False):
+                  p_drop=0.0, seed=0, dtype=np.float64, return_probs=False, pos_offset=(0, 0, 0)):
 	"""O [B,Sq,Hq,D] and LSE [B,Hq,Sq] (natural log) of exact attention.
 
 	q [B,Sq,Hq,D], k/v [B,Sk,Hkv,D].  Rows with no allowed key give O = 0 and
@@ -181,17 +203,17 @@ def attention_fwd(q, k, v, bias=None, causal=False, scale=None, seqlens=None,
 		lse = np.where(l[..., 0] > 0, np.log(np.where(l > 0, l, 1.0))[..., 0] + m_safe[..., 0], -np.inf)
 	pd = p
 	if p_drop > 0.0:
-		keep = dropout_keep_mask(seed, p_drop, B, Hq, Sq, Sk)
+		keep = dropout_keep_mask(seed, p_drop, B, Hq, Sq, Sk, pos_offset)
 		pd = np.where(keep, p, 0.0) / dtype(1.0 - float(np.float32(p_drop)))
 	vf = np.repeat(np.asarray(v, dtype=dtype), r, axis=2)
-	o = np.einsum("bhij,bjhd->bihd", pd, vf)
+	o = _pv(pd, vf)
 	if return_probs:
 		return o, lse, p, pd
 	return o, lse
 
 
 def attention_bwd(q, k, v, dO, bias=None, causal=False, scale=None, seqlens=None,
-                  p_drop=0.0, seed=0, dtype=np.float64):
+                  p_drop=0.0, seed=0, dtype=np.float64, pos_offset=(0, 0, 0)):
 	"""Analytic gradients (dQ, dK, dV) of sum(O * dO); FlashAttention-2 Algorithm 2,
 	the same five products as flash_attention_jax/_backward_jax.py:111-127, with
 	dK/dV summed over the q-heads of each KV group (_backward_triton.py:1156-1161).
@@ -199,23 +221,23 @@ def attention_bwd(q, k, v, dO, bias=None, causal=False, scale=None, seqlens=None
 	B, Sq, Hq, D = q.shape
 	Sk, Hkv = k.shape[1], k.shape[2]
 	scale = (1.0 / math.sqrt(D)) if scale is None else scale
-	o, lse, p, pd = attention_fwd(q, k, v, bias, causal, scale, seqlens, p_drop, seed, dtype, True)
+	o, lse, p, pd = attention_fwd(q, k, v, bias, causal, scale, seqlens, p_drop, seed, dtype, True, pos_offset)
 	r = Hq // Hkv
 	dOf = np.asarray(dO, dtype=dtype)
 	qf = np.asarray(q, dtype=dtype)
 	kf = np.repeat(np.asarray(k, dtype=dtype), r, axis=2)
 	vf = np.repeat(np.asarray(v, dtype=dtype), r, axis=2)
-	dv_full = np.einsum("bhij,bihd->bjhd", pd, dOf)
-	dpd = np.einsum("bihd,bjhd->bhij", dOf, vf)
+	dv_full = _ptx(pd, dOf)
+	dpd = _qk(dOf, vf)
 	if p_drop > 0.0:
-		keep = dropout_keep_mask(seed, p_drop, B, Hq, Sq, Sk)
+		keep = dropout_keep_mask(seed, p_drop, B, Hq, Sq, Sk, pos_offset)
 		dp = np.where(keep, dpd, 0.0) / dtype(1.0 - float(np.float32(p_drop)))
 	else:
 		dp = dpd
 	delta = np.einsum("bihd,bihd->bhi", o, dOf)[..., None]  # = rowsum(P * dP)
 	ds = p * (dp - delta)
-	dq = np.einsum("bhij,bjhd->bihd", ds, kf) * dtype(scale)
-	dk_full = np.einsum("bhij,bihd->bjhd", ds, qf) * dtype(scale)
+	dq = _pv(ds, kf) * dtype(scale)
+	dk_full = _ptx(ds, qf) * dtype(scale)
 	dk = dk_full.reshape(B, Sk, Hkv, r, D).sum(axis=3)
 	dv = dv_full.reshape(B, Sk, Hkv, r, D).sum(axis=3)
 	return dq, dk, dv

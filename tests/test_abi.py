@@ -1,0 +1,130 @@
+"""The C ABI without a GPU: the library loads, exports every symbol that
+include/fa2.h declares, the ctypes mirror of fa2_params has the C layout, and
+argument validation returns the documented codes.  No kernel is launched."""
+
+import ctypes
+import os
+import re
+import subprocess
+import sys
+import tempfile
+
+import pytest
+
+from jax_flash_attn2 import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "fa2.h")
+
+
+def _declared_functions():
+	src = open(HEADER).read()
+	src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+	return sorted(set(re.findall(r"\b(fa2_[a-z_0-9]+)\s*\(", src)))
+
+
+def test_library_exports_every_declared_symbol():
+	lib = _lib.load()
+	names = _declared_functions()
+	assert set(names) == set(_lib.EXPORTS)
+	for n in names:
+		assert hasattr(lib, n), n
+	assert lib.fa2_version() >= 100
+
+
+def test_struct_layout_matches_c():
+	prog = r"""
+#include <stdio.h>
+#include <stddef.h>
+#include "fa2.h"
+int main(void) {
+  printf("%zu %zu %zu %zu %zu %zu %zu %zu %zu\n", sizeof(fa2_params), offsetof(fa2_params, seed), offsetof(fa2_params, q),
+         offsetof(fa2_params, lse), offsetof(fa2_params, bias), offsetof(fa2_params, bias_stride_b),
+         offsetof(fa2_params, seqlens), offsetof(fa2_params, dout), offsetof(fa2_params, scratch));
+  return 0;
+}"""
+	with tempfile.TemporaryDirectory() as d:
+		c = os.path.join(d, "t.c")
+		open(c, "w").write(prog)
+		exe = os.path.join(d, "t")
+		subprocess.check_call(["gcc", "-I", os.path.join(ROOT, "include"), c, "-o", exe])
+		got = [int(x) for x in subprocess.check_output([exe]).split()]
+	P = _lib.Fa2Params
+	want = [ctypes.sizeof(P)] + [getattr(P, f).offset for f in ("seed", "q", "lse", "bias", "bias_stride_b", "seqlens", "dout", "scratch")]
+	assert got == want
+
+
+def _good_params():
+	p = _lib.new_params()
+	p.dtype = _lib.FA2_BF16
+	p.B, p.Sq, p.Sk, p.Hq, p.Hkv, p.D = 2, 128, 128, 8, 2, 128
+	p.scale = 0.088
+	for name in ("q", "k", "v", "o", "dout", "dq", "dk", "dv"):
+		t = getattr(p, name)
+		t.ptr = 0x10000
+		t.stride_b, t.stride_s, t.stride_h = 128 * 8 * 128, 8 * 128, 128
+	p.lse = 0x20000
+	p.scratch = 0x30000
+	p.scratch_bytes = 1 << 20
+	return p
+
+
+def _rc(p, which=0):
+	return _lib.load().fa2_validate(ctypes.byref(p), which)
+
+
+def test_validate_accepts_good_params():
+	p = _good_params()
+	assert _rc(p, 0) == 0 and _rc(p, 1) == 0
+	assert _lib.load().fa2_bwd_scratch_bytes(ctypes.byref(p)) == 2 * 8 * 128 * 4
+
+
+@pytest.mark.parametrize(
+	"mutate,code",
+	[
+		(lambda p: setattr(p, "struct_size", 8), -1),
+		(lambda p: setattr(p, "dtype", 3), -2),  # fp32 q/k/v: "Only support fp16 and bf16"
+		(lambda p: setattr(p, "Sq", 0), -3),
+		(lambda p: setattr(p, "Hkv", 3), -4),
+		(lambda p: setattr(p.q, "ptr", 0), -5),
+		(lambda p: setattr(p.k, "ptr", 0x10008), -5),
+		(lambda p: setattr(p.v, "stride_s", 1028), -6),
+		(lambda p: setattr(p, "p_drop", 1.0), -7),
+		(lambda p: setattr(p, "p_drop", -0.1), -7),
+		(lambda p: (setattr(p, "bias", 0x40000), setattr(p, "bias_dtype", 7)), -8),
+		(lambda p: (setattr(p, "bias", 0x40000), setattr(p, "bias_dtype", 2), setattr(p, "bias_stride_m", 64)), -8),
+		(lambda p: (setattr(p, "seqlens", 0x50000), setattr(p, "Sk", 256)), -9),
+		(lambda p: (setattr(p, "seqlens", 0x50000), setattr(p, "bias", 0x40000), setattr(p, "bias_dtype", 2),
+		            setattr(p, "bias_stride_m", 128)), -9),
+		(lambda p: setattr(p, "D", 96), -10),
+	],
+)
+def test_validate_error_codes(mutate, code):
+	p = _good_params()
+	mutate(p)
+	assert _rc(p, 0) == code
+	assert _lib.strerror(code) != "unknown error"
+
+
+def test_validate_backward_scratch():
+	p = _good_params()
+	p.scratch_bytes = 16
+	assert _rc(p, 1) == -11 and _rc(p, 0) == 0
+	p = _good_params()
+	p.scratch = 0
+	assert _rc(p, 1) == -11
+	p = _good_params()
+	p.dq.ptr = 0
+	assert _rc(p, 1) == -5
+	lib = _lib.load()
+	# errors never reach a launch: NULL stream and bogus pointers are fine here
+	assert lib.fa2_bwd(ctypes.byref(p), None) == -5
+	assert lib.fa2_fwd(None, None) == -1
+	assert lib.fa2_dropout_mask(ctypes.byref(p), None, None) == -5
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+	monkeypatch.setattr(_lib, "_lib", None)
+	monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libfa2_hip.so")
+	with pytest.raises(ImportError):
+		_lib.load()

@@ -1,0 +1,131 @@
+"""The five benchmark configurations at FULL size on the GPU.
+
+The NumPy oracle cannot evaluate S x S score matrices for every (batch, head)
+of these shapes in seconds, so each config is checked (a) against the oracle
+on slices that are self-contained - whole KV groups of one batch row, or the
+last rows / last keys of a causal problem - and (b) through size-independent
+properties (probabilities sum to one through LSE, V = 1 gives O = 1,
+delta identity, GQA reduction).
+"""
+
+import numpy as np
+import pytest
+import torch
+
+import fa2_oracle as O
+from _cases import TOL_GRAD_REL_L2, TOL_O, check_forward, check_grads
+from jax_flash_attn2 import _hip_op as op
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _gen(shape, seed, mul, dtype):
+	g = torch.Generator(device=DEV).manual_seed(seed)
+	return (torch.randn(shape, generator=g, device=DEV, dtype=torch.float32) * mul).to(dtype)
+
+
+def _np(t):
+	return t.float().cpu().numpy().astype(np.float32)
+
+
+def _check_group(q, k, v, do, o, lse, grads, b, g, r, dtype, **kw):
+	"""Oracle on batch row b, KV head g with its r query heads: self-contained for O, LSE, dQ, dK, dV."""
+	hs = slice(g * r, (g + 1) * r)
+	args = [_np(q[b:b + 1, :, hs]), _np(k[b:b + 1, :, g:g + 1]), _np(v[b:b + 1, :, g:g + 1])]
+	kw = dict(kw, dtype=np.float32, pos_offset=(b, g * r, 0))
+	o_ref, lse_ref = O.attention_fwd(*args, **kw)
+	check_forward(o[b:b + 1, :, hs], lse[b:b + 1, hs], o_ref, lse_ref, dtype, f"group b{b} g{g}")
+	if grads is not None:
+		g_ref = O.attention_bwd(*args, _np(do[b:b + 1, :, hs]), **kw)
+		got = (grads[0][b:b + 1, :, hs], grads[1][b:b + 1, :, g:g + 1], grads[2][b:b + 1, :, g:g + 1])
+		check_grads(got, g_ref, f"group b{b} g{g}")
+
+
+def test_c1_readme_shape_fp16_causal_forward():
+	# B2 Hq16 Hkv4 S512 D64 fp16 causal, forward only, N(0,1) inputs
+	dtype = torch.float16
+	q, k, v = _gen((2, 512, 16, 64), 0, 1.0, dtype), _gen((2, 512, 4, 64), 1, 1.0, dtype), _gen((2, 512, 4, 64), 2, 1.0, dtype)
+	o, lse = op.fwd(q, k, v, causal=True)
+	o_ref, lse_ref = O.attention_fwd(_np(q), _np(k), _np(v), causal=True)
+	check_forward(o, lse, o_ref, lse_ref, dtype, "c1")
+
+
+def test_c2_llama_prefill_bf16_causal_fwd_bwd():
+	# B4 S4096 Hq32 Hkv8 D128 bf16 causal
+	dtype = torch.bfloat16
+	B, S, Hq, Hkv, D = 4, 4096, 32, 8, 128
+	q, k, v = _gen((B, S, Hq, D), 0, 0.5, dtype), _gen((B, S, Hkv, D), 1, 0.5, dtype), _gen((B, S, Hkv, D), 2, 0.5, dtype)
+	do = _gen((B, S, Hq, D), 3, 1.0, dtype)
+	o, lse = op.fwd(q, k, v, causal=True)
+	grads = op.bwd(q, k, v, o, lse, do, causal=True)
+	for b, g in ((0, 0), (3, 7)):
+		_check_group(q, k, v, do, o, lse, grads, b, g, 4, dtype, causal=True)
+	# V = 1 -> O = 1 for every (b, h, i)
+	o1, _ = op.fwd(q, k, torch.ones_like(v), causal=True)
+	assert (o1.float() - 1).abs().max().item() <= 1e-2
+	for t in grads:
+		assert torch.isfinite(t.float()).all()
+
+
+def test_c3_padded_mha_bias_bf16_fwd_bwd():
+	# B8 S2048 H16 D64 bf16 non-causal, bias [B,1,S,S] = 1/(1+|i-j|) + finfo.min on padded keys
+	dtype = torch.bfloat16
+	B, S, H, D = 8, 2048, 16, 64
+	q, k, v = _gen((B, S, H, D), 0, 0.5, dtype), _gen((B, S, H, D), 1, 0.5, dtype), _gen((B, S, H, D), 2, 0.5, dtype)
+	do = _gen((B, S, H, D), 3, 1.0, dtype)
+	i = torch.arange(S, device=DEV)
+	base = 1.0 / (1.0 + (i[:, None] - i[None, :]).abs().float())
+	lens = torch.randint(S // 2, S + 1, (B,), generator=torch.Generator().manual_seed(4))
+	valid = i[None, :] < lens.to(DEV)[:, None]
+	bias = torch.where(valid[:, None, None, :], base[None, None], torch.tensor(torch.finfo(dtype).min, device=DEV)).to(dtype)
+	o, lse = op.fwd(q, k, v, bias)
+	grads = op.bwd(q, k, v, o, lse, do, bias)
+	for b, h in ((0, 0), (7, 15), (3, 5)):
+		_check_group(q, k, v, do, o, lse, grads, b, h, 1, dtype, bias=_np(bias[b:b + 1]))
+	# masked keys receive exactly zero gradient
+	for b in range(B):
+		L = int(lens[b])
+		if L < S:
+			assert grads[1][b, L:].abs().max().item() == 0 and grads[2][b, L:].abs().max().item() == 0
+
+
+def test_c4_long_context_bf16_causal_fwd_bwd():
+	# B1 S32768 Hq64 Hkv8 D128 bf16 causal.  Oracle on the last 256 rows (all keys) of one KV group:
+	# exact for O, LSE, dQ of those rows, and for dK, dV of the last 256 keys (only those rows see them).
+	dtype = torch.bfloat16
+	B, S, Hq, Hkv, D = 1, 32768, 64, 8, 128
+	q, k, v = _gen((B, S, Hq, D), 0, 0.5, dtype), _gen((B, S, Hkv, D), 1, 0.5, dtype), _gen((B, S, Hkv, D), 2, 0.5, dtype)
+	do = _gen((B, S, Hq, D), 3, 1.0, dtype)
+	o, lse = op.fwd(q, k, v, causal=True)
+	dq, dk, dv = op.bwd(q, k, v, o, lse, do, causal=True)
+	R = 256
+	for g in (0, 7):
+		hs = slice(g * 8, (g + 1) * 8)
+		args = [_np(q[:, S - R:, hs]), _np(k[:, :, g:g + 1]), _np(v[:, :, g:g + 1])]
+		o_ref, lse_ref = O.attention_fwd(*args, causal=True, dtype=np.float32)
+		check_forward(o[:, S - R:, hs], lse[:, hs, S - R:], o_ref, lse_ref, dtype, f"c4 g{g}")
+		dq_ref, dk_ref, dv_ref = O.attention_bwd(*args, _np(do[:, S - R:, hs]), causal=True, dtype=np.float32)
+		check_grads((dq[:, S - R:, hs], dk[:, S - R:, g:g + 1], dv[:, S - R:, g:g + 1]),
+		            (dq_ref, dk_ref[:, S - R:], dv_ref[:, S - R:]), f"c4 g{g}")
+	# first rows: row 0 attends to key 0 only -> O[0] = V[0], LSE = scale q0.k0
+	assert torch.equal(o[0, 0].reshape(8, 8, D), v[0, 0][:, None, :].expand(8, 8, D))
+	# V = 1 -> O = 1 everywhere (every row tile, every causal tile boundary)
+	o1, _ = op.fwd(q, k, torch.ones_like(v), causal=True)
+	assert (o1.float() - 1).abs().max().item() <= 1e-2
+	assert torch.isfinite(dq.float()).all() and torch.isfinite(dk.float()).all() and torch.isfinite(dv.float()).all()
+
+
+def test_c5_dropout_wide_heads_bf16_causal_fwd_bwd():
+	# B8 S2048 H16 D256 bf16 causal, dropout 0.1, seed 42
+	dtype = torch.bfloat16
+	B, S, H, D = 8, 2048, 16, 256
+	q, k, v = _gen((B, S, H, D), 0, 0.5, dtype), _gen((B, S, H, D), 1, 0.5, dtype), _gen((B, S, H, D), 2, 0.5, dtype)
+	do = _gen((B, S, H, D), 3, 1.0, dtype)
+	o, lse = op.fwd(q, k, v, None, None, None, 0.1, True, 42)
+	grads = op.bwd(q, k, v, o, lse, do, None, None, None, 0.1, True, 42)
+	for b, h in ((0, 0), (7, 15)):
+		_check_group(q, k, v, do, o, lse, grads, b, h, 1, dtype, causal=True, p_drop=0.1, seed=42)
+	# LSE does not depend on dropout
+	_, lse0 = op.fwd(q, k, v, causal=True)
+	assert torch.equal(lse, lse0)

@@ -1,0 +1,223 @@
+"""Pins the CPU oracle: known-answer vectors, closed forms, invariants, finite
+differences and the committed golden fixtures.  No GPU."""
+
+import os
+
+import numpy as np
+import pytest
+import scipy.special
+
+import fa2_oracle as O
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def _hex(words):
+	return " ".join("%08x" % int(x) for x in words)
+
+
+# Random123 kat_vectors, philox4x32 with 10 rounds
+@pytest.mark.parametrize(
+	"ctr,key,expect",
+	[
+		((0, 0, 0, 0), (0, 0), "6627e8d5 e169c58d bc57ac4c 9b00dbd8"),
+		((0xFFFFFFFF,) * 4, (0xFFFFFFFF,) * 2, "408f276d 41c83b0e a20bc7c6 6d5451fd"),
+		((0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344), (0xA4093822, 0x299F31D0), "d16cfe09 94fdcceb 5001e420 24126ea1"),
+	],
+)
+def test_philox_known_answers(ctr, key, expect):
+	assert _hex(O.philox4x32_10(*[np.uint32(c) for c in ctr], *key)) == expect
+
+
+def test_dropout_mask_definition_and_rate():
+	B, H, Sq, Sk, p, seed = 2, 3, 37, 50, 0.25, (7 << 32) | 12345
+	keep = O.dropout_keep_mask(seed, p, B, H, Sq, Sk)
+	thr = O.dropout_threshold(p)
+	assert thr == 1 << 30
+	# spot-check single elements against a scalar evaluation of the definition
+	for (b, h, i, j) in [(0, 0, 0, 0), (1, 2, 36, 49), (0, 1, 5, 6), (1, 0, 20, 3)]:
+		w = O.philox4x32_10(np.uint32(j >> 2), np.uint32(i), np.uint32(h), np.uint32(b), seed & 0xFFFFFFFF, seed >> 32)
+		assert bool(keep[b, h, i, j]) == (int(w[j & 3]) >= thr)
+	big = O.dropout_keep_mask(42, 0.1, 1, 2, 512, 512)
+	n = big.size
+	assert abs(big.mean() - 0.9) < 4 * np.sqrt(0.09 / n)
+	# slices of a larger problem reproduce through pos_offset
+	sl = O.dropout_keep_mask(seed, p, 1, 1, 7, Sk, pos_offset=(1, 2, 30))
+	assert np.array_equal(sl[0, 0], keep[1, 2, 30:37])
+	assert O.dropout_keep_mask(1, 0.0, 1, 1, 8, 8).all()
+
+
+def _rand(rng, B, Sq, Sk, Hq, Hkv, D):
+	return (rng.normal(size=(B, Sq, Hq, D)), rng.normal(size=(B, Sk, Hkv, D)), rng.normal(size=(B, Sk, Hkv, D)),
+	        rng.normal(size=(B, Sq, Hq, D)))
+
+
+def test_forward_matches_scipy_softmax():
+	rng = np.random.default_rng(1)
+	q, k, v, _ = _rand(rng, 2, 9, 11, 4, 4, 8)
+	bias = rng.normal(size=(2, 4, 9, 11))
+	o, lse = O.attention_fwd(q, k, v, bias=bias, scale=0.3)
+	s = np.einsum("bihd,bjhd->bhij", q, k) * 0.3 + bias
+	p = scipy.special.softmax(s, axis=-1)
+	assert np.allclose(o, np.einsum("bhij,bjhd->bihd", p, v), atol=1e-12)
+	assert np.allclose(lse, scipy.special.logsumexp(s, axis=-1), atol=1e-12)
+
+
+def test_forward_invariants():
+	rng = np.random.default_rng(2)
+	q, k, v, _ = _rand(rng, 2, 16, 16, 4, 2, 8)
+	# V = 1 -> O = 1
+	o, _ = O.attention_fwd(q, k, np.ones_like(v), causal=True)
+	assert np.allclose(o, 1.0)
+	# Q = 0, causal -> prefix mean of V (per kv group)
+	o, _ = O.attention_fwd(np.zeros_like(q), k, v, causal=True)
+	pm = np.cumsum(v, axis=1) / np.arange(1, 17)[None, :, None, None]
+	assert np.allclose(o, np.repeat(pm, 2, axis=2))
+	# key permutation leaves O unchanged without a causal mask
+	perm = rng.permutation(16)
+	o1, l1 = O.attention_fwd(q, k, v)
+	o2, l2 = O.attention_fwd(q, k[:, perm], v[:, perm])
+	assert np.allclose(o1, o2) and np.allclose(l1, l2)
+	# a per-row constant in the bias does not change O and shifts LSE
+	c = rng.normal(size=(2, 4, 16, 1))
+	o3, l3 = O.attention_fwd(q, k, v, bias=np.broadcast_to(c, (2, 4, 16, 16)))
+	assert np.allclose(o1, o3) and np.allclose(l3, l1 + c[..., 0])
+	# GQA == MHA over repeated K/V, q-head h -> kv-head h // r
+	o4, _ = O.attention_fwd(q, np.repeat(k, 2, axis=2), np.repeat(v, 2, axis=2))
+	assert np.allclose(o1, o4)
+
+
+def test_causal_alignment_and_fully_masked_rows():
+	rng = np.random.default_rng(3)
+	# Sq > Sk: rows i < Sq - Sk see no key -> zeros and LSE = -inf (bottom-right aligned)
+	q, k, v, _ = _rand(rng, 1, 6, 4, 2, 2, 4)
+	o, lse = O.attention_fwd(q, k, v, causal=True)
+	assert np.all(o[:, :2] == 0) and np.all(np.isneginf(lse[:, :, :2]))
+	ok = O.allowed_mask(1, 6, 4, True)[0]
+	assert np.array_equal(ok, np.arange(4)[None, :] <= np.arange(6)[:, None] - 2)
+	# Sq < Sk: row i sees keys <= i + (Sk - Sq)
+	assert np.array_equal(O.allowed_mask(1, 2, 5, True)[0], np.array([[1, 1, 1, 1, 0], [1, 1, 1, 1, 1]], bool))
+	# seqlens: keys beyond len masked, padded rows zero
+	q, k, v, _ = _rand(rng, 2, 8, 8, 2, 2, 4)
+	o, lse = O.attention_fwd(q, k, v, seqlens=[5, 8])
+	o5, _ = O.attention_fwd(q[:1, :5], k[:1, :5], v[:1, :5])
+	assert np.allclose(o[0, :5], o5[0]) and np.all(o[0, 5:] == 0)
+
+
+def test_bias_broadcast_rules():
+	rng = np.random.default_rng(4)
+	B, S, Hq, Hkv, D = 2, 8, 4, 2, 4
+	q, k, v, _ = _rand(rng, B, S, S, Hq, Hkv, D)
+	full = rng.normal(size=(B, Hq, S, S))
+	for shape in [(1, 1), (B, 1), (1, Hq), (B, Hq)]:
+		b = full[: shape[0], : shape[1]]
+		o1, _ = O.attention_fwd(q, k, v, bias=b)
+		o2, _ = O.attention_fwd(q, k, v, bias=np.broadcast_to(b, (B, Hq, S, S)))
+		assert np.allclose(o1, o2)
+	bg = full[:, :Hkv]
+	o1, _ = O.attention_fwd(q, k, v, bias=bg)
+	o2, _ = O.attention_fwd(q, k, v, bias=np.repeat(bg, 2, axis=1))
+	assert np.allclose(o1, o2)
+	with pytest.raises(ValueError):
+		O.attention_fwd(q, k, v, bias=full[:, :3])
+	with pytest.raises(ValueError):
+		O.attention_fwd(q, k, v, bias=full[..., :7])
+	# mask -> finfo.min bias equals boolean masking when each row keeps a key
+	valid = np.arange(S)[None, :] < np.array([5, 8])[:, None]
+	mb = np.broadcast_to(np.where(valid[:, None, None, :], 0.0, np.finfo(np.float32).min), (2, 1, S, S))
+	o3, _ = O.attention_fwd(q, k, v, bias=mb)
+	o4, _ = O.attention_fwd(q[:1], k[:1, :5], v[:1, :5])
+	assert np.allclose(o3[0], o4[0])
+
+
+@pytest.mark.parametrize(
+	"kw",
+	[dict(), dict(causal=True), dict(bias=True), dict(causal=True, p_drop=0.3, seed=7), dict(seqlens=[5, 6]),
+	 dict(causal=True, scale=0.7)],
+)
+def test_backward_matches_finite_differences(kw):
+	rng = np.random.default_rng(5)
+	B, Sq, Sk, Hq, Hkv, D = 2, 6, 6, 4, 2, 4
+	q, k, v, dO = _rand(rng, B, Sq, Sk, Hq, Hkv, D)
+	kw = dict(kw)
+	if kw.get("bias") is True:
+		kw["bias"] = rng.normal(size=(B, Hkv, Sq, Sk))
+	grads = O.attention_bwd(q, k, v, dO, **kw)
+	f = lambda *a: np.sum(O.attention_fwd(*a, **kw)[0] * dO)
+	eps = 1e-6
+	for idx, g in enumerate(grads):
+		xs = [q, k, v]
+		num = np.zeros_like(xs[idx])
+		it = np.nditer(xs[idx], flags=["multi_index"])
+		for _ in it:
+			mi = it.multi_index
+			a = [t.copy() for t in xs]
+			b = [t.copy() for t in xs]
+			a[idx][mi] += eps
+			b[idx][mi] -= eps
+			num[mi] = (f(*a) - f(*b)) / (2 * eps)
+		assert np.abs(num - g).max() < 1e-7
+
+
+def test_backward_identities():
+	rng = np.random.default_rng(6)
+	q, k, v, dO = _rand(rng, 1, 12, 12, 4, 2, 8)
+	o, lse, p, _ = O.attention_fwd(q, k, v, causal=True, return_probs=True)
+	assert np.allclose(p.sum(-1), 1.0)
+	# delta = rowsum(dO * O) = rowsum(P * dP)
+	vf = np.repeat(v, 2, axis=2)
+	dp = np.einsum("bihd,bjhd->bhij", dO, vf)
+	assert np.allclose(np.einsum("bihd,bihd->bhi", o, dO), (p * dp).sum(-1))
+	# dK/dV of a group = sum of the MHA gradients over its q-heads
+	dq, dk, dv = O.attention_bwd(q, k, v, dO, causal=True)
+	dq2, dk2, dv2 = O.attention_bwd(q, np.repeat(k, 2, axis=2), vf, dO, causal=True)
+	assert np.allclose(dq, dq2)
+	assert np.allclose(dk, dk2.reshape(1, 12, 2, 2, 8).sum(3)) and np.allclose(dv, dv2.reshape(1, 12, 2, 2, 8).sum(3))
+
+
+def test_blockwise_restatement_equals_closed_form():
+	rng = np.random.default_rng(7)
+	B, S, Hq, Hkv, D = 1, 256, 4, 2, 16
+	q, k, v, dO = _rand(rng, B, S, S, Hq, Hkv, D)
+	bias = rng.normal(size=(B, 1, S, S))
+	o, (dq, dk, dv) = O.jax_platform_call(q, k, v, bias=bias, dtype=np.float64, with_grads_for=dO, blocksize_q=64, blocksize_k=128)
+	o2, _ = O.attention_fwd(q, k, v, bias=bias)
+	g2 = O.attention_bwd(q, k, v, dO, bias=bias)
+	assert np.abs(o - o2).max() < 1e-6
+	for a, b in zip((dq, dk, dv), g2):
+		assert np.abs(a - b).max() < 1e-5
+	# with a mask the reference also skips blocks above the diagonal
+	qt, kt, vt = (np.ascontiguousarray(np.swapaxes(x, 1, 2)) for x in (q, np.repeat(k, 2, 2), np.repeat(v, 2, 2)))
+	tri = np.tril(np.ones((S, S), bool))[None, None]
+	ob, lse = O.blockwise_fwd(qt / 4.0, kt, vt, mask=tri, dtype=np.float64, blocksize_q=64, blocksize_k=64)
+	oc, _ = O.attention_fwd(q, k, v, causal=True)
+	assert np.abs(np.swapaxes(ob, 1, 2) - oc).max() < 1e-6
+
+
+def test_bf16_helpers_round_trip():
+	x = np.array([1.0, 1.00390625, 1.005859375, -3.3895314e38, 65504.0, 1e-40], np.float32)
+	r = O.round_bf16(x)
+	assert r[0] == 1.0 and r[1] == 1.0 and r[2] == 1.0078125  # ties-to-even, then up
+	assert np.array_equal(O.from_bf16_bits(O.to_bf16_bits(r)), r)
+
+
+@pytest.mark.parametrize("name", sorted(f for f in os.listdir(os.path.join(HERE, "golden")) if f.endswith(".npz")))
+def test_golden_fixtures(name):
+	"""The committed fixtures (made by tests/golden/make_golden.py from this oracle) still reproduce."""
+	z = np.load(os.path.join(HERE, "golden", name))
+	kw = dict(causal=bool(z["causal"]), p_drop=float(z["p_drop"]), seed=int(z["seed"]))
+	if "bias" in z:
+		kw["bias"] = z["bias"]
+	if "seqlens" in z:
+		kw["seqlens"] = z["seqlens"]
+	o, lse = O.attention_fwd(z["q"], z["k"], z["v"], **kw)
+	dq, dk, dv = O.attention_bwd(z["q"], z["k"], z["v"], z["dout"], **kw)
+	fin = np.isfinite(z["lse"])
+	assert np.allclose(o, z["o"], atol=1e-6) and np.allclose(lse[fin], z["lse"][fin], atol=1e-6)
+	assert np.array_equal(np.isfinite(lse), fin)
+	for a, b in ((dq, z["dq"]), (dk, z["dk"]), (dv, z["dv"])):
+		assert np.allclose(a, b, atol=1e-6)
+	if float(z["p_drop"]) > 0:
+		B, Sq, Hq, _ = z["q"].shape
+		keep = O.dropout_keep_mask(int(z["seed"]), float(z["p_drop"]), B, Hq, Sq, z["k"].shape[1])
+		assert np.array_equal(np.unpackbits(z["keep_bits"])[: keep.size].astype(bool).reshape(keep.shape), keep)

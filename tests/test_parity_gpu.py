@@ -1,0 +1,256 @@
+"""GPU parity: the HIP path, called through the C ABI of libfa2_hip.so,
+against the NumPy oracle on the same seeded inputs.
+
+Tolerances (BASELINE north star): max-abs error on O <= 2e-2 (bf16) / 5e-3
+(fp16) and relative L2 error on dQ/dK/dV <= 1e-2, against an fp64/fp32
+evaluation; the dropout keep-mask is bit-exact.
+"""
+
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import fa2_oracle as O
+from _cases import TOL_O, check_forward, check_grads, f64, make_inputs
+from jax_flash_attn2 import _hip_op as op
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def _dev(t):
+	return None if t is None else t.to(DEV)
+
+
+def _run_case(B, Sq, Sk, Hq, Hkv, D, dtype, causal=False, bias_shape=None, p=0.0, seed=0, seqlens=None, scale=None,
+              bias_dtype=None, data_seed=0):
+	q, k, v, do, bias = make_inputs(B, Sq, Sk, Hq, Hkv, D, dtype, data_seed, bias_shape, bias_dtype=bias_dtype)
+	sl = None if seqlens is None else torch.tensor(seqlens, dtype=torch.int32)
+	kw = dict(causal=causal, p_drop=p, seed=seed, seqlens=seqlens, scale=scale)
+	o_ref, lse_ref = O.attention_fwd(f64(q), f64(k), f64(v), f64(bias), **kw)
+	g_ref = O.attention_bwd(f64(q), f64(k), f64(v), f64(do), f64(bias), **kw)
+	o, lse = op.fwd(_dev(q), _dev(k), _dev(v), _dev(bias), _dev(sl), scale, p, causal, seed)
+	g = op.bwd(_dev(q), _dev(k), _dev(v), o, lse, _dev(do), _dev(bias), _dev(sl), scale, p, causal, seed)
+	torch.cuda.synchronize()
+	what = f"B{B} Sq{Sq} Sk{Sk} Hq{Hq} Hkv{Hkv} D{D} {dtype} causal={causal} bias={bias_shape} p={p} seqlens={seqlens}"
+	check_forward(o, lse, o_ref, lse_ref, dtype, what)
+	check_grads(g, g_ref, what)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("D", [64, 128, 256])
+@pytest.mark.parametrize("causal", [False, True])
+def test_basic_shapes(dtype, D, causal):
+	_run_case(2, 320, 320, 4, 2, D, dtype, causal=causal)
+
+
+@pytest.mark.parametrize(
+	"Sq,Sk",
+	[(1, 1), (1, 77), (7, 5), (33, 33), (63, 65), (128, 128), (129, 257), (257, 129), (200, 333), (500, 64), (64, 500)],
+)
+@pytest.mark.parametrize("causal", [False, True])
+def test_ragged_and_cross_lengths(Sq, Sk, causal):
+	"""Ragged tiles, Sq != Sk with the bottom-right aligned causal mask, rows without any allowed key."""
+	_run_case(2, Sq, Sk, 4, 2, 128, torch.bfloat16, causal=causal)
+	_run_case(1, Sq, Sk, 2, 1, 64, torch.float16, causal=causal, data_seed=1)
+
+
+@pytest.mark.parametrize("r", [1, 2, 4, 8])
+def test_gqa_group_sizes(r):
+	_run_case(2, 192, 192, 8, 8 // r, 128, torch.bfloat16, causal=True)
+	_run_case(1, 130, 130, 8, 8 // r, 64, torch.bfloat16, causal=False, data_seed=2)
+
+
+@pytest.mark.parametrize(
+	"bshape", [(1, 1), (2, 1), (1, 4), (2, 4), (2, 2)], ids=["b1h1", "bBh1", "b1hH", "bBhH", "bBhKV"]
+)
+@pytest.mark.parametrize("D", [64, 128])
+def test_bias_broadcast(bshape, D):
+	B, Sq, Sk, Hq, Hkv = 2, 160, 224, 4, 2
+	_run_case(B, Sq, Sk, Hq, Hkv, D, torch.bfloat16, causal=False, bias_shape=(*bshape, Sq, Sk))
+	_run_case(B, Sq, Sk, Hq, Hkv, D, torch.bfloat16, causal=True, bias_shape=(*bshape, Sq, Sk), data_seed=3)
+
+
+def test_bias_dtypes_and_unaligned_rows():
+	# fp32 bias with a 16-bit q; odd Sk makes bias rows unaligned for vector loads
+	_run_case(1, 70, 75, 2, 2, 64, torch.float16, bias_shape=(1, 2, 70, 75), bias_dtype=torch.float32)
+	_run_case(1, 70, 75, 2, 2, 128, torch.bfloat16, bias_shape=(1, 1, 70, 75), bias_dtype=torch.float16, causal=True)
+	_run_case(1, 96, 96, 2, 2, 256, torch.bfloat16, bias_shape=(1, 2, 96, 96))
+
+
+def test_mask_as_finfo_min_bias():
+	"""Boolean mask -> where(mask, 0, finfo.min) bias (the README recipe) must equal key-length masking."""
+	B, S, H, D = 2, 192, 4, 64
+	dtype = torch.bfloat16
+	q, k, v, do, _ = make_inputs(B, S, S, H, H, D, dtype, 5)
+	lens = [100, 192]
+	valid = torch.arange(S)[None, :] < torch.tensor(lens)[:, None]
+	i = torch.arange(S)
+	base = 1.0 / (1.0 + (i[:, None] - i[None, :]).abs().float())
+	bias = torch.where(valid[:, None, None, :], base[None, None], torch.tensor(torch.finfo(dtype).min)).to(dtype)
+	o_ref, lse_ref = O.attention_fwd(f64(q), f64(k), f64(v), f64(bias))
+	g_ref = O.attention_bwd(f64(q), f64(k), f64(v), f64(do), f64(bias))
+	o, lse = op.fwd(_dev(q), _dev(k), _dev(v), _dev(bias))
+	g = op.bwd(_dev(q), _dev(k), _dev(v), o, lse, _dev(do), _dev(bias))
+	check_forward(o, lse, o_ref, lse_ref, dtype, "finfo.min bias")
+	check_grads(g, g_ref, "finfo.min bias")
+	# masked keys get exactly zero gradient
+	assert g[1][0, 100:].abs().max().item() == 0 and g[2][0, 100:].abs().max().item() == 0
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_seqlens(causal):
+	_run_case(4, 256, 256, 4, 2, 128, torch.bfloat16, causal=causal, seqlens=[256, 100, 1, 0])
+	_run_case(3, 200, 200, 2, 2, 64, torch.float16, causal=causal, seqlens=[17, 200, 129])
+
+
+@pytest.mark.parametrize("D", [64, 128, 256])
+def test_dropout(D):
+	_run_case(2, 192, 192, 4, 2, D, torch.bfloat16, causal=True, p=0.1, seed=42)
+	_run_case(1, 100, 150, 2, 2, D, torch.float16, causal=False, p=0.5, seed=(9 << 32) | 5, data_seed=4)
+
+
+def test_custom_softmax_scale():
+	_run_case(1, 128, 128, 2, 2, 128, torch.bfloat16, causal=True, scale=0.2)
+
+
+@pytest.mark.parametrize(
+	"name", sorted(f[:-4] for f in os.listdir(os.path.join(HERE, "golden")) if f.endswith(".npz"))
+)
+def test_golden_fixtures(name):
+	z = np.load(os.path.join(HERE, "golden", name + ".npz"))
+	dtype = torch.bfloat16  # fixture inputs are bf16-representable
+	t = lambda a: torch.from_numpy(np.asarray(a)).to(dtype).to(DEV)
+	causal, p, seed = bool(z["causal"]), float(z["p_drop"]), int(z["seed"])
+	bias = t(z["bias"]) if "bias" in z else None
+	sl = torch.from_numpy(z["seqlens"]).to(DEV) if "seqlens" in z else None
+	o, lse = op.fwd(t(z["q"]), t(z["k"]), t(z["v"]), bias, sl, None, p, causal, seed)
+	g = op.bwd(t(z["q"]), t(z["k"]), t(z["v"]), o, lse, t(z["dout"]), bias, sl, None, p, causal, seed)
+	check_forward(o, lse, z["o"], z["lse"], dtype, name)
+	check_grads(g, (z["dq"], z["dk"], z["dv"]), name)
+	if p > 0:
+		B, Sq, Hq, _ = z["q"].shape
+		Sk = z["k"].shape[1]
+		keep = op.dropout_mask(B, Hq, Sq, Sk, p, seed, DEV).cpu().numpy().astype(bool)
+		want = np.unpackbits(z["keep_bits"])[: keep.size].astype(bool).reshape(keep.shape)
+		assert np.array_equal(keep, want)
+
+
+@pytest.mark.parametrize(
+	"B,H,Sq,Sk,p,seed",
+	[(2, 3, 37, 50, 0.25, 12345), (1, 2, 128, 129, 0.1, 42), (1, 1, 5, 3, 0.9, (1 << 63) | 7), (3, 1, 64, 256, 0.5, 0),
+	 (1, 2, 16, 16, 0.0, 99)],
+)
+def test_dropout_mask_is_bit_exact(B, H, Sq, Sk, p, seed):
+	keep = op.dropout_mask(B, H, Sq, Sk, p, seed, DEV).cpu().numpy().astype(bool)
+	assert np.array_equal(keep, O.dropout_keep_mask(seed, p, B, H, Sq, Sk))
+
+
+def test_kernels_apply_exactly_the_exported_mask():
+	"""Read the mask back out of each kernel: with q = 0 the probabilities are uniform,
+	and one-hot V / dO / K rows turn O, dV and dQ into scaled copies of the keep-mask."""
+	B, H, S, D, p, seed = 2, 2, 64, 64, 0.3, 4242
+	dtype = torch.float16
+	eye = torch.eye(S, D, dtype=dtype, device=DEV)[None, :, None, :].expand(B, S, H, D).contiguous()
+	zero = torch.zeros(B, S, H, D, dtype=dtype, device=DEV)
+	ones = torch.ones(B, S, H, D, dtype=dtype, device=DEV)
+	keep = O.dropout_keep_mask(seed, p, B, H, S, S)  # [B,H,i,j]
+	inv = 1.0 / (1.0 - float(np.float32(p)))
+	# forward: O[b,i,h,j] = keep[b,h,i,j] / (S (1-p))
+	o, lse = op.fwd(zero, eye, eye, None, None, None, p, False, seed)
+	got = (o.float().permute(0, 2, 1, 3).cpu().numpy() * S / inv) > 0.5
+	assert np.array_equal(got, keep)
+	# dK/dV kernel: dO one-hot -> dV[b,j,h,i] = keep[b,h,i,j] / (S (1-p))
+	dq, dk, dv = op.bwd(zero, eye, eye, o, lse, eye, None, None, None, p, False, seed)
+	got = (dv.float().permute(0, 2, 3, 1).cpu().numpy() * S / inv) > 0.5
+	assert np.array_equal(got, keep)
+	# dQ kernel: K, V one-hot, dO = 1 -> dQ[b,i,h,j] = scale/S (keep/(1-p) - delta_i)
+	dq, dk, dv = op.bwd(zero, eye, eye, o, lse, ones, None, None, None, p, False, seed)
+	delta = (o.float() * 1.0).sum(-1, keepdim=True)
+	rec = dq.float() * S * (D ** 0.5) + delta
+	got = (rec.permute(0, 2, 1, 3).cpu().numpy() / inv) > 0.5
+	assert np.array_equal(got, keep)
+
+
+def test_backward_is_deterministic_and_outputs_fully_written():
+	q, k, v, do, _ = make_inputs(2, 300, 300, 8, 2, 128, torch.bfloat16, 7)
+	q, k, v, do = (_dev(t) for t in (q, k, v, do))
+	o, lse = op.fwd(q, k, v, causal=True)
+	a = op.bwd(q, k, v, o, lse, do, causal=True)
+	b = op.bwd(q, k, v, o, lse, do, causal=True)
+	for x, y in zip(a, b):
+		assert torch.equal(x, y)
+	# poison-filled outputs: every element must be overwritten
+	plan = op.Plan(q, k, v, dout=do, causal=True)
+	for t in (plan.out, plan.dq, plan.dk, plan.dv):
+		t.fill_(float("nan"))
+	plan.lse.fill_(float("nan"))
+	plan.forward()
+	plan.backward()
+	torch.cuda.synchronize()
+	for t in (plan.out, plan.lse, plan.dq, plan.dk, plan.dv):
+		assert torch.isfinite(t.float()).all()
+	assert torch.equal(plan.dq, a[0]) and torch.equal(plan.dk, a[1]) and torch.equal(plan.dv, a[2])
+
+
+def test_strided_inputs_from_a_fused_qkv_buffer():
+	B, S, Hq, Hkv, D = 2, 160, 4, 2, 128
+	dtype = torch.bfloat16
+	g = torch.Generator().manual_seed(11)
+	fused = (torch.randn(B, S, Hq + 2 * Hkv, D, generator=g) * 0.5).to(dtype)
+	do = torch.randn(B, S, Hq, D, generator=g).to(dtype)
+	q, k, v = fused[:, :, :Hq], fused[:, :, Hq:Hq + Hkv], fused[:, :, Hq + Hkv:]
+	o_ref, lse_ref = O.attention_fwd(f64(q), f64(k), f64(v), causal=True)
+	g_ref = O.attention_bwd(f64(q), f64(k), f64(v), f64(do), causal=True)
+	fd = fused.to(DEV)
+	qd, kd, vd = fd[:, :, :Hq], fd[:, :, Hq:Hq + Hkv], fd[:, :, Hq + Hkv:]
+	assert not qd.is_contiguous()
+	o, lse = op.fwd(qd, kd, vd, causal=True)
+	gr = op.bwd(qd, kd, vd, o, lse, _dev(do), causal=True)
+	check_forward(o, lse, o_ref, lse_ref, dtype, "strided")
+	check_grads(gr, g_ref, "strided")
+
+
+def test_gqa_equals_mha_on_repeated_kv():
+	q, k, v, do, _ = make_inputs(1, 256, 256, 8, 2, 128, torch.bfloat16, 8)
+	q, k, v, do = (_dev(t) for t in (q, k, v, do))
+	o1, l1 = op.fwd(q, k, v, causal=True)
+	kr, vr = k.repeat_interleave(4, dim=2), v.repeat_interleave(4, dim=2)
+	o2, l2 = op.fwd(q, kr, vr, causal=True)
+	assert torch.equal(o1, o2) and torch.equal(l1, l2)
+	g1 = op.bwd(q, k, v, o1, l1, do, causal=True)
+	g2 = op.bwd(q, kr, vr, o2, l2, do, causal=True)
+	assert torch.equal(g1[0], g2[0])
+	for a, b in ((g1[1], g2[1]), (g1[2], g2[2])):
+		ref = b.float().reshape(1, 256, 2, 4, 128).sum(3)
+		assert O.rel_l2(a.float().cpu().numpy(), ref.cpu().numpy()) < 5e-3
+
+
+def test_facade_forward_and_autograd():
+	"""FlashAttention(AttentionConfig(...)).forward / __call__ with gradients through the operator."""
+	from jax_flash_attn2 import AttentionConfig, Backend, FlashAttention, Platform
+
+	attn = FlashAttention(AttentionConfig(platform=Platform.HIP, backend=Backend.GPU))
+	q, k, v, do, bias = make_inputs(2, 128, 128, 4, 2, 64, torch.bfloat16, 9, bias_shape=(2, 2, 128, 128))
+	qd, kd, vd = (_dev(t).requires_grad_() for t in (q, k, v))
+	out = attn.forward(qd, kd, vd, bias=_dev(bias), causal=True, dropout_prob=0.1, dropout_seed=7)
+	out.backward(_dev(do))
+	kw = dict(causal=True, p_drop=0.1, seed=7)
+	o_ref, _ = O.attention_fwd(f64(q), f64(k), f64(v), f64(bias), **kw)
+	g_ref = O.attention_bwd(f64(q), f64(k), f64(v), f64(do), f64(bias), **kw)
+	assert np.abs(out.detach().float().cpu().numpy() - o_ref).max() <= TOL_O[torch.bfloat16]
+	check_grads((qd.grad, kd.grad, vd.grad), g_ref, "facade")
+	# 2-D padding mask, Sq == Sk; with Sq != Sk the mask is dropped and a single row is never causal
+	mask = (torch.arange(128)[None, :] < torch.tensor([128, 50])[:, None]).to(DEV)
+	o2 = attn(qd.detach(), kd.detach(), vd.detach(), attention_mask=mask)
+	o2_ref, _ = O.attention_fwd(f64(q), f64(k), f64(v), seqlens=[128, 50])
+	assert np.abs(o2.float().cpu().numpy() - o2_ref).max() <= TOL_O[torch.bfloat16]
+	o3 = attn(qd.detach()[:, :1], kd.detach(), vd.detach(), attention_mask=mask, causal=True)
+	o3_ref, _ = O.attention_fwd(f64(q)[:, :1], f64(k), f64(v), causal=False)
+	assert np.abs(o3.float().cpu().numpy() - o3_ref).max() <= TOL_O[torch.bfloat16]
+	with pytest.warns(UserWarning):
+		o4 = FlashAttention(AttentionConfig(platform=Platform.TRITON, backend=Backend.GPU))(qd.detach(), kd.detach(), vd.detach())
+	assert torch.equal(o4, attn(qd.detach(), kd.detach(), vd.detach()))
