@@ -37,7 +37,7 @@ enum {
 	FA2_OK = 0,
 	FA2_EINVAL_STRUCT = -1,   /* NULL params or struct_size too small            */
 	FA2_EINVAL_DTYPE = -2,    /* q/k/v dtype not fp16/bf16 (_forward_triton.py:494-495) */
-	FA2_EINVAL_SHAPE = -3,    /* non-positive dimension                          */
+	FA2_EINVAL_SHAPE = -3,    /* non-positive dimension, or scale not finite and > 0 */
 	FA2_EINVAL_HEADS = -4,    /* Hq % Hkv != 0 (flash_attention.py:189-193)      */
 	FA2_EINVAL_PTR = -5,      /* required pointer is NULL or not 16-byte aligned */
 	FA2_EINVAL_STRIDE = -6,   /* stride not a multiple of 8 elements             */
@@ -63,7 +63,7 @@ typedef struct fa2_params {
 	int32_t B, Sq, Sk, Hq, Hkv, D;
 	int32_t causal;         /* bottom-right aligned: j <= i + Sk - Sq
 	                           (_forward_triton.py:127-132)                */
-	float scale;            /* softmax scale, applied to q.k^T             */
+	float scale;            /* softmax scale, applied to q.k^T; must be > 0 */
 	float p_drop;           /* dropout probability in [0,1)                */
 	uint64_t seed;          /* Philox key for the dropout keep-mask        */
 

@@ -40,7 +40,7 @@ int validate(const fa2_params* p, int which) {
 	if (p->Hq % p->Hkv) return FA2_EINVAL_HEADS;
 	if (p->D != 64 && p->D != 128 && p->D != 256) return FA2_EUNSUPPORTED;
 	if (!(p->p_drop >= 0.f && p->p_drop < 1.f)) return FA2_EINVAL_DROPOUT;
-	if (!isfinite(p->scale)) return FA2_EINVAL_SHAPE;
+	if (!isfinite(p->scale) || !(p->scale > 0.f)) return FA2_EINVAL_SHAPE;
 	int rc;
 	if ((rc = check_tensor(p->q, true))) return rc;
 	if ((rc = check_tensor(p->k, true))) return rc;
@@ -188,7 +188,7 @@ const char* fa2_strerror(int code) {
 		case FA2_OK: return "ok";
 		case FA2_EINVAL_STRUCT: return "params is NULL or struct_size is smaller than sizeof(fa2_params)";
 		case FA2_EINVAL_DTYPE: return "Only support fp16 and bf16";
-		case FA2_EINVAL_SHAPE: return "dimensions must be positive and scale finite";
+		case FA2_EINVAL_SHAPE: return "dimensions must be positive and the softmax scale finite and positive";
 		case FA2_EINVAL_HEADS: return "query heads must be divisible by key/value heads";
 		case FA2_EINVAL_PTR: return "required pointer is NULL or misaligned";
 		case FA2_EINVAL_STRIDE: return "batch/sequence/head strides must be multiples of 8 elements";

@@ -173,6 +173,135 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		}
 	};
 
+	// per-lane LDS byte offsets (swizzle folded in) of the fragments read in the loop
+	int poff[KS];
+#pragma unroll
+	for (int ks = 0; ks < KS; ++ks) poff[ks] = tile_off<D>(c, 2 * ks + g);
+	int toff[DB][2];
+	{
+		int i16 = lane & 15;
+		int trow = 4 * g + (i16 >> 2);
+		int tcol = 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
+#pragma unroll
+		for (int db = 0; db < DB; ++db) {
+			int col = 32 * db + tcol;
+			toff[db][0] = tile_off<D>(trow, col >> 3) + ((col & 4) << 1);
+			toff[db][1] = tile_off<D>(trow + 8, col >> 3) + ((col & 4) << 1);
+		}
+	}
+
+	// One streamed tile of BMQ query rows of q-head hq.  MASKED = some (row, key)
+	// of this wave's 32 keys x BMQ rows is masked.
+	auto tile_body = [&](auto masked_tag, int buf, int hq, int m0) {
+		constexpr bool MASKED = decltype(masked_tag)::value;
+		const FA2_LDS char* qt = lds + buf * TILE_BYTES;
+		const FA2_LDS char* dot = lds + (2 + buf) * TILE_BYTES;
+		const FA2_LDS char* lse_s = stat + buf * STAT_BYTES;
+		const FA2_LDS char* del_s = stat + (2 + buf) * STAT_BYTES;
+		const char* bias_base = nullptr;
+		if constexpr (BIAS) {
+			int hb = a.bias_group ? hk : hq;
+			int jc = jcol < a.Sk ? jcol : a.Sk - 1;
+			int es = a.bias_dtype == 3 ? 4 : 2;
+			bias_base = a.bias + (int64_t)b * a.bias_sb + (int64_t)hb * a.bias_sh + (int64_t)jc * es;
+		}
+#pragma unroll 1
+		for (int qb = 0; qb < QB; ++qb) {
+			// bias column for this lane's key, 16 rows
+			float bv[BIAS ? 16 : 1];
+			if constexpr (BIAS) {
+#pragma unroll
+				for (int i = 0; i < 16; ++i) {
+					int row = m0 + 32 * qb + 8 * (i >> 2) + 4 * g + (i & 3);
+					row = row < a.Sq ? row : a.Sq - 1;
+					const char* pp = bias_base + (int64_t)row * a.bias_sm;
+					bv[i] = a.bias_dtype == 3 ? *(const float*)pp
+					        : a.bias_dtype == 2 ? (float)*(const __bf16*)pp
+					                            : (float)*(const _Float16*)pp;
+				}
+			}
+			f32x16 s, dp;
+#pragma unroll
+			for (int i = 0; i < 16; ++i) s[i] = dp[i] = 0.f;
+#pragma unroll
+			for (int ks = 0; ks < KS; ++ks) {
+				V8 qa = *(const FA2_LDS V8*)(qt + poff[ks] + qb * (32 * D * 2));
+				s = mfma32(qa, kf[ks], s);
+			}
+#pragma unroll
+			for (int ks = 0; ks < KS; ++ks) {
+				V8 da = *(const FA2_LDS V8*)(dot + poff[ks] + qb * (32 * D * 2));
+				dp = mfma32(da, vf[ks], dp);
+			}
+			// transposed fragments for the two products below, one batch per 16-row half:
+			// issued early so that their LDS latency is covered by the products above and
+			// by the elementwise math
+			constexpr bool BOTH_EARLY = DB <= 4;
+			u32x4 tfr[2][2 * DB];
+			const uint32_t dot_a = lds_addr(dot) + qb * (32 * D * 2);
+			const uint32_t qt_a = lds_addr(qt) + qb * (32 * D * 2);
+			auto issue_t = [&](int hf, u32x4(&dst)[2 * DB]) {
+#pragma unroll
+				for (int db = 0; db < DB; ++db) {
+					dst[2 * db] = lds_tr_issue_rt<D>(dot_a + toff[db][0], dot_a + toff[db][1], hf);
+					dst[2 * db + 1] = lds_tr_issue_rt<D>(qt_a + toff[db][0], qt_a + toff[db][1], hf);
+				}
+			};
+			issue_t(0, tfr[0]);
+			if constexpr (BOTH_EARLY) issue_t(1, tfr[1]);
+			f32x4 lse4[4], del4[4];
+#pragma unroll
+			for (int aa = 0; aa < 4; ++aa) {
+				lse4[aa] = *(const FA2_LDS f32x4*)(lse_s + (32 * qb + 8 * aa + 4 * g) * 4);
+				del4[aa] = *(const FA2_LDS f32x4*)(del_s + (32 * qb + 8 * aa + 4 * g) * 4);
+			}
+			__builtin_amdgcn_sched_barrier(0);
+			f32x16 pd;  // P after dropout (feeds dV); s becomes dS (feeds dK)
+#pragma unroll
+			for (int i = 0; i < 16; ++i) {
+				int row = m0 + 32 * qb + 8 * (i >> 2) + 4 * g + (i & 3);
+				float lse = lse4[i >> 2][i & 3], del = del4[i >> 2][i & 3];
+				float p;
+				if constexpr (BIAS)
+					p = exp2_fast((__builtin_fmaf(s[i], c1, bv[i]) - lse) * kLog2e);
+				else
+					p = exp2_fast(__builtin_fmaf(s[i], c1, -lse));
+				if constexpr (MASKED) {
+					bool ok = row < sq_eff && jcol < sk_eff && (!a.causal || jcol <= row + off);
+					p = ok ? p : 0.f;
+				}
+				float pdrop = p, dpe = dp[i];
+				if constexpr (DROP) {
+					u32x4 rnd = philox4x32_10((uint32_t)(jcol >> 2), (uint32_t)row, (uint32_t)hq, (uint32_t)b, a.drop_k0, a.drop_k1);
+					uint32_t word = rnd[0];
+					word = (jcol & 3) == 1 ? rnd[1] : word;
+					word = (jcol & 3) == 2 ? rnd[2] : word;
+					word = (jcol & 3) == 3 ? rnd[3] : word;
+					bool keep = word >= a.drop_thr;
+					pdrop = keep ? p : 0.f;
+					dpe = keep ? dpe * a.drop_inv_keep : 0.f;
+				}
+				pd[i] = pdrop;
+				s[i] = p * (dpe - del);
+			}
+			// dV^T += dO^T P ; dK^T += Q^T dS   (k runs over the tile's 32 rows, two steps of 16)
+#pragma unroll
+			for (int hf = 0; hf < 2; ++hf) {
+				V8 pb = pack8<T>(pd[8 * hf + 0], pd[8 * hf + 1], pd[8 * hf + 2], pd[8 * hf + 3], pd[8 * hf + 4], pd[8 * hf + 5],
+				                 pd[8 * hf + 6], pd[8 * hf + 7]);
+				V8 sb = pack8<T>(s[8 * hf + 0], s[8 * hf + 1], s[8 * hf + 2], s[8 * hf + 3], s[8 * hf + 4], s[8 * hf + 5],
+				                 s[8 * hf + 6], s[8 * hf + 7]);
+				if (hf == 0 || !BOTH_EARLY) lds_tr_wait(tfr[hf]);
+				if (hf == 0 && !BOTH_EARLY) issue_t(1, tfr[1]);
+#pragma unroll
+				for (int db = 0; db < DB; ++db) {
+					dv[db] = mfma32(as_frag<T>(tfr[hf][2 * db]), pb, dv[db]);
+					dk[db] = mfma32(as_frag<T>(tfr[hf][2 * db + 1]), sb, dk[db]);
+				}
+			}
+		}
+	};
+
 	if (steps > 0) {
 		issue_tile(0, 0);
 		store_stat(fetch_stat(0), 0);
@@ -185,7 +314,9 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		float next_stat = 0.f;
 		const bool has_next = step + 1 < steps;
 		if (has_next) {
+#ifndef FA2_DBG_NOLOAD
 			issue_tile(step + 1, buf ^ 1);
+#endif
 			next_stat = fetch_stat(step + 1);
 		}
 		const int hq = hk * r + step / nq;
@@ -193,97 +324,15 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		// wave-uniform: any work / any masking for (rows m0.., keys wn0..)?
 		int last_row = m0 + BMQ - 1 < sq_eff - 1 ? m0 + BMQ - 1 : sq_eff - 1;
 		bool skip = wn0 >= sk_eff || (a.causal && wn0 > last_row + off);
+#ifdef FA2_DBG_NOCOMPUTE
+		skip = true;
+#endif
 		if (!skip) {
 			const bool need_mask = (m0 + BMQ > sq_eff) || (wn0 + 32 > sk_eff) || (a.causal && wn0 + 31 > m0 + off);
-			const FA2_LDS char* qt = lds + buf * TILE_BYTES;
-			const FA2_LDS char* dot = lds + (2 + buf) * TILE_BYTES;
-			const FA2_LDS char* lse_s = stat + buf * STAT_BYTES;
-			const FA2_LDS char* del_s = stat + (2 + buf) * STAT_BYTES;
-			const char* bias_base = nullptr;
-			if constexpr (BIAS) {
-				int hb = a.bias_group ? hk : hq;
-				int jc = jcol < a.Sk ? jcol : a.Sk - 1;
-				int es = a.bias_dtype == 3 ? 4 : 2;
-				bias_base = a.bias + (int64_t)b * a.bias_sb + (int64_t)hb * a.bias_sh + (int64_t)jc * es;
-			}
-#pragma unroll
-			for (int qb = 0; qb < QB; ++qb) {
-				// bias column for this lane's key, 16 rows
-				float bv[BIAS ? 16 : 1];
-				if constexpr (BIAS) {
-#pragma unroll
-					for (int i = 0; i < 16; ++i) {
-						int row = m0 + 32 * qb + 8 * (i >> 2) + 4 * g + (i & 3);
-						row = row < a.Sq ? row : a.Sq - 1;
-						const char* pp = bias_base + (int64_t)row * a.bias_sm;
-						bv[i] = a.bias_dtype == 3 ? *(const float*)pp
-						        : a.bias_dtype == 2 ? (float)*(const __bf16*)pp
-						                            : (float)*(const _Float16*)pp;
-					}
-				}
-				f32x16 s, dp;
-#pragma unroll
-				for (int i = 0; i < 16; ++i) s[i] = dp[i] = 0.f;
-#pragma unroll
-				for (int ks = 0; ks < KS; ++ks) {
-					V8 qa = lds_frag<T, D>(qt, 32 * qb, ks, lane);
-					s = mfma32(qa, kf[ks], s);
-				}
-#pragma unroll
-				for (int ks = 0; ks < KS; ++ks) {
-					V8 da = lds_frag<T, D>(dot, 32 * qb, ks, lane);
-					dp = mfma32(da, vf[ks], dp);
-				}
-				f32x4 lse4[4], del4[4];
-#pragma unroll
-				for (int aa = 0; aa < 4; ++aa) {
-					lse4[aa] = *(const FA2_LDS f32x4*)(lse_s + (32 * qb + 8 * aa + 4 * g) * 4);
-					del4[aa] = *(const FA2_LDS f32x4*)(del_s + (32 * qb + 8 * aa + 4 * g) * 4);
-				}
-				f32x16 pd;  // P after dropout (feeds dV); s becomes dS (feeds dK)
-#pragma unroll
-				for (int i = 0; i < 16; ++i) {
-					int row = m0 + 32 * qb + 8 * (i >> 2) + 4 * g + (i & 3);
-					float lse = lse4[i >> 2][i & 3], del = del4[i >> 2][i & 3];
-					float p;
-					if constexpr (BIAS)
-						p = exp2_fast((__builtin_fmaf(s[i], c1, bv[i]) - lse) * kLog2e);
-					else
-						p = exp2_fast(__builtin_fmaf(s[i], c1, -lse));
-					if (need_mask) {
-						bool ok = row < sq_eff && jcol < sk_eff && (!a.causal || jcol <= row + off);
-						p = ok ? p : 0.f;
-					}
-					float pdrop = p, dpe = dp[i];
-					if constexpr (DROP) {
-						u32x4 rnd = philox4x32_10((uint32_t)(jcol >> 2), (uint32_t)row, (uint32_t)hq, (uint32_t)b, a.drop_k0, a.drop_k1);
-						uint32_t word = rnd[0];
-						word = (jcol & 3) == 1 ? rnd[1] : word;
-						word = (jcol & 3) == 2 ? rnd[2] : word;
-						word = (jcol & 3) == 3 ? rnd[3] : word;
-						bool keep = word >= a.drop_thr;
-						pdrop = keep ? p : 0.f;
-						dpe = keep ? dpe * a.drop_inv_keep : 0.f;
-					}
-					pd[i] = pdrop;
-					s[i] = p * (dpe - del);
-				}
-				// dV^T += dO^T P ; dK^T += Q^T dS   (k runs over the tile's 32 rows, two steps of 16)
-#pragma unroll
-				for (int hf = 0; hf < 2; ++hf) {
-					V8 pb = pack8<T>(pd[8 * hf + 0], pd[8 * hf + 1], pd[8 * hf + 2], pd[8 * hf + 3], pd[8 * hf + 4], pd[8 * hf + 5],
-					                 pd[8 * hf + 6], pd[8 * hf + 7]);
-					V8 sb = pack8<T>(s[8 * hf + 0], s[8 * hf + 1], s[8 * hf + 2], s[8 * hf + 3], s[8 * hf + 4], s[8 * hf + 5],
-					                 s[8 * hf + 6], s[8 * hf + 7]);
-#pragma unroll
-					for (int db = 0; db < DB; ++db) {
-						V8 dot_a = lds_frag_tr<T, D>(dot, 32 * qb + 16 * hf, 32 * db, lane);
-						dv[db] = mfma32(dot_a, pb, dv[db]);
-						V8 qt_a = lds_frag_tr<T, D>(qt, 32 * qb + 16 * hf, 32 * db, lane);
-						dk[db] = mfma32(qt_a, sb, dk[db]);
-					}
-				}
-			}
+			if (need_mask)
+				tile_body(std::true_type{}, buf, hq, m0);
+			else
+				tile_body(std::false_type{}, buf, hq, m0);
 		}
 		if (has_next) store_stat(next_stat, buf ^ 1);
 	}
@@ -426,22 +475,24 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_kernel(const KArgs a) {
 		bias_base = a.bias + (int64_t)b * a.bias_sb + (int64_t)hb * a.bias_sh;
 	}
 
-	for (int t = 0; t < ntiles; ++t) {
-		const int n0 = t * BN;
-		const int buf = t & 1;
-		wait_async_loads();
-		__syncthreads();
-		if (t + 1 < ntiles) {
-			int n1 = n0 + BN;
-			int rows = sk_eff - n1 < BN ? sk_eff - n1 : BN;
-			tile_load_async<D, BN, NT>(lds + (buf ^ 1) * TILE_BYTES, kbase + (int64_t)n1 * a.k.ss, a.k.ss, rows, tid);
-			tile_load_async<D, BN, NT>(lds + (2 + (buf ^ 1)) * TILE_BYTES, vbase + (int64_t)n1 * a.v.ss, a.v.ss, rows, tid);
+	int koff[KS];
+#pragma unroll
+	for (int ks = 0; ks < KS; ++ks) koff[ks] = tile_off<D>(c, 2 * ks + g);
+	int toff[DB][2];
+	{
+		int i16 = lane & 15;
+		int trow = 4 * g + (i16 >> 2);
+		int tcol = 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
+#pragma unroll
+		for (int db = 0; db < DB; ++db) {
+			int col = 32 * db + tcol;
+			toff[db][0] = tile_off<D>(trow, col >> 3) + ((col & 4) << 1);
+			toff[db][1] = tile_off<D>(trow + 8, col >> 3) + ((col & 4) << 1);
 		}
-		if (n0 > wave_jmax) continue;
-		const bool need_mask = n0 + BN - 1 > wave_jmin;
-		const FA2_LDS char* kt = lds + buf * TILE_BYTES;
-		const FA2_LDS char* vt = lds + (2 + buf) * TILE_BYTES;
+	}
 
+	auto tile_body = [&](auto masked_tag, const FA2_LDS char* kt, const FA2_LDS char* vt, int n0) {
+		constexpr bool MASKED = decltype(masked_tag)::value;
 #pragma unroll
 		for (int kb = 0; kb < KB; ++kb) {
 			f32x4 bv[BIAS ? QB : 1][4];
@@ -462,16 +513,26 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_kernel(const KArgs a) {
 				for (int i = 0; i < 16; ++i) s[qb][i] = dp[qb][i] = 0.f;
 #pragma unroll
 			for (int ks = 0; ks < KS; ++ks) {
-				V8 ka = lds_frag<T, D>(kt, 32 * kb, ks, lane);
+				V8 ka = *(const FA2_LDS V8*)(kt + koff[ks] + kb * (32 * D * 2));
 #pragma unroll
 				for (int qb = 0; qb < QB; ++qb) s[qb] = mfma32(ka, qf[qb][ks], s[qb]);
 			}
 #pragma unroll
 			for (int ks = 0; ks < KS; ++ks) {
-				V8 va = lds_frag<T, D>(vt, 32 * kb, ks, lane);
+				V8 va = *(const FA2_LDS V8*)(vt + koff[ks] + kb * (32 * D * 2));
 #pragma unroll
 				for (int qb = 0; qb < QB; ++qb) dp[qb] = mfma32(va, dof[qb][ks], dp[qb]);
 			}
+			// K^T fragments for dQ^T += K^T dS^T, issued ahead of the elementwise math
+			constexpr bool BOTH_EARLY = DB <= 4;
+			u32x4 kfr[2][DB];
+			const uint32_t kt_a = lds_addr(kt) + kb * (32 * D * 2);
+			auto issue_k = [&](int hf, u32x4(&dst)[DB]) {
+#pragma unroll
+				for (int db = 0; db < DB; ++db) dst[db] = lds_tr_issue_rt<D>(kt_a + toff[db][0], kt_a + toff[db][1], hf);
+			};
+			issue_k(0, kfr[0]);
+			if constexpr (BOTH_EARLY) issue_k(1, kfr[1]);
 			V8 dsf[QB][2];
 #pragma unroll
 			for (int qb = 0; qb < QB; ++qb) {
@@ -490,7 +551,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_kernel(const KArgs a) {
 							p = exp2_fast((__builtin_fmaf(s[qb][i], c1, bv[qb][aa][e]) - lse_r[qb]) * kLog2e);
 						else
 							p = exp2_fast(__builtin_fmaf(s[qb][i], c1, -lse_r[qb]));
-						if (need_mask) {
+						if constexpr (MASKED) {
 							int j = n0 + 32 * kb + 8 * aa + 4 * g + e;
 							p = j <= jmax[qb] ? p : 0.f;
 						}
@@ -508,14 +569,35 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_kernel(const KArgs a) {
 			}
 			// dQ^T += K^T dS^T
 #pragma unroll
-			for (int hf = 0; hf < 2; ++hf)
+			for (int hf = 0; hf < 2; ++hf) {
+				if (hf == 0 || !BOTH_EARLY) lds_tr_wait(kfr[hf]);
+				if (hf == 0 && !BOTH_EARLY) issue_k(1, kfr[1]);
 #pragma unroll
-				for (int db = 0; db < DB; ++db) {
-					V8 kta = lds_frag_tr<T, D>(kt, 32 * kb + 16 * hf, 32 * db, lane);
+				for (int db = 0; db < DB; ++db)
 #pragma unroll
-					for (int qb = 0; qb < QB; ++qb) dq[qb][db] = mfma32(kta, dsf[qb][hf], dq[qb][db]);
-				}
+					for (int qb = 0; qb < QB; ++qb) dq[qb][db] = mfma32(as_frag<T>(kfr[hf][db]), dsf[qb][hf], dq[qb][db]);
+			}
 		}
+	};
+
+	for (int t = 0; t < ntiles; ++t) {
+		const int n0 = t * BN;
+		const int buf = t & 1;
+		wait_async_loads();
+		__syncthreads();
+		if (t + 1 < ntiles) {
+			int n1 = n0 + BN;
+			int rows = sk_eff - n1 < BN ? sk_eff - n1 : BN;
+			tile_load_async<D, BN, NT>(lds + (buf ^ 1) * TILE_BYTES, kbase + (int64_t)n1 * a.k.ss, a.k.ss, rows, tid);
+			tile_load_async<D, BN, NT>(lds + (2 + (buf ^ 1)) * TILE_BYTES, vbase + (int64_t)n1 * a.v.ss, a.v.ss, rows, tid);
+		}
+		if (n0 > wave_jmax) continue;
+		const FA2_LDS char* kt = lds + buf * TILE_BYTES;
+		const FA2_LDS char* vt = lds + (2 + buf) * TILE_BYTES;
+		if (n0 + BN - 1 > wave_jmin)
+			tile_body(std::true_type{}, kt, vt, n0);
+		else
+			tile_body(std::false_type{}, kt, vt, n0);
 	}
 
 	char* obase = a.dq.ptr + (int64_t)b * a.dq.sb + (int64_t)h * a.dq.sh;
@@ -545,8 +627,8 @@ struct BwdCfg {
 	static constexpr int KV_QB = D <= 128 ? 2 : 1;
 	static constexpr int KV_BN = KV_NW * 32;
 	// dQ: 4 waves x QB x 32 rows
-	static constexpr int DQ_NW = 4;
-	static constexpr int DQ_QB = D <= 64 ? 2 : 1;
+	static constexpr int DQ_NW = D <= 128 ? 8 : 4;
+	static constexpr int DQ_QB = 1;
 	static constexpr int DQ_BM = DQ_NW * DQ_QB * 32;
 };
 

@@ -13,12 +13,16 @@
 // softmax needs only in-lane reductions plus one exchange with lane l^32, and
 // rescaling O is a multiply by a per-lane scalar.
 #pragma once
+#include <type_traits>
+
 #include "fa2_common.hpp"
 #include "fa2_kernels.hpp"
 
 namespace fa2 {
 
 constexpr int kFwdBN = 64;
+// the running row maximum is only raised when exceeded by more than this (log2 units)
+constexpr float kRescaleSlack = 8.f;
 
 // blockIdx.x -> (row tile, q-head, batch).  With xcd_remap the workgroups of
 // one (batch, kv-head) - which share K and V - are kept on one XCD (hardware
@@ -190,22 +194,29 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const KArgs a) {
 		bias_base = a.bias + (int64_t)b * a.bias_sb + (int64_t)hb * a.bias_sh;
 	}
 
-	for (int t = 0; t < ntiles; ++t) {
-		const int n0 = t * BN;
-		const int buf = t & 1;
-		wait_async_loads();
-		__syncthreads();
-		if (t + 1 < ntiles) {
-			int n1 = n0 + BN;
-			int rows = sk_eff - n1 < BN ? sk_eff - n1 : BN;
-			tile_load_async<D, BN, NT>(lds + (buf ^ 1) * TILE_BYTES, kbase + (int64_t)n1 * a.k.ss, a.k.ss, rows, tid);
-			tile_load_async<D, BN, NT>(lds + (2 + (buf ^ 1)) * TILE_BYTES, vbase + (int64_t)n1 * a.v.ss, a.v.ss, rows, tid);
+	// Per-lane LDS byte offsets with the swizzle folded in, so that every fragment
+	// read in the loop is base + register + immediate.
+	//   K fragment (ks):      row c (+32 kb), chunk 2ks+g
+	//   V fragment (kk, db):  rows 16kk + 4g + (lane&15)/4 (+8), 8 bytes at column 32db + 16((lane>>4)&1) + 4(lane&3)
+	int koff[KS];
+#pragma unroll
+	for (int ks = 0; ks < KS; ++ks) koff[ks] = tile_off<D>(c, 2 * ks + g);
+	int voff[DB][2];
+	{
+		int i16 = lane & 15;
+		int vrow = 4 * g + (i16 >> 2);
+		int vcol = 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
+#pragma unroll
+		for (int db = 0; db < DB; ++db) {
+			int col = 32 * db + vcol;
+			voff[db][0] = tile_off<D>(vrow, col >> 3) + ((col & 4) << 1);
+			voff[db][1] = tile_off<D>(vrow + 8, col >> 3) + ((col & 4) << 1);
 		}
-		if (n0 > wave_jmax) continue;  // whole tile masked for this wave (uniform)
-		const bool need_mask = n0 + BN - 1 > wave_jmin;
-		const FA2_LDS char* kt = lds + buf * TILE_BYTES;
-		const FA2_LDS char* vt = lds + (2 + buf) * TILE_BYTES;
+	}
 
+	// One K/V tile.  MASKED = some element of the tile is masked for this wave.
+	auto tile_body = [&](auto masked_tag, const FA2_LDS char* kt, const FA2_LDS char* vt, int n0) {
+		constexpr bool MASKED = decltype(masked_tag)::value;
 		// bias tile, fetched ahead of the matrix products
 		f32x4 bv[BIAS ? KB : 1][BIAS ? QB : 1][4];
 		if constexpr (BIAS) {
@@ -233,12 +244,34 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const KArgs a) {
 		for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
 			for (int kb = 0; kb < KB; ++kb) {
-				V8 kf = lds_frag<T, D>(kt, 32 * kb, ks, lane);
+				V8 kf = *(const FA2_LDS V8*)(kt + koff[ks] + kb * (32 * D * 2));
 #pragma unroll
 				for (int qb = 0; qb < QB; ++qb) s[kb][qb] = mfma32(kf, qf[qb][ks], s[kb][qb]);
 			}
 
-		// online softmax, one query row per lane
+		// V fragments for O^T += V^T P^T, fetched in batches of NF; the first batch is in
+		// flight during the softmax, each further one during the products of the previous.
+		constexpr int KK = BN / 16;
+		constexpr int FPB = (8 / DB) < 1 ? 1 : ((8 / DB) > KK ? KK : (8 / DB));  // 16-key steps per batch
+		constexpr int NBATCH = KK / FPB;
+		constexpr int NF = FPB * DB;
+		u32x4 vfr[2][NF];
+		const uint32_t vt_a = lds_addr(vt);
+		auto issue_v = [&](auto batch_tag, u32x4(&dst)[NF]) {
+			constexpr int BI = decltype(batch_tag)::value;
+#pragma unroll
+			for (int f = 0; f < FPB; ++f)
+#pragma unroll
+				for (int db = 0; db < DB; ++db) {
+					dst[f * DB + db] = lds_tr_issue_rt<D>(vt_a + voff[db][0], vt_a + voff[db][1], BI * FPB + f);
+				}
+		};
+		issue_v(std::integral_constant<int, 0>{}, vfr[0]);
+
+		// online softmax, one query row per lane.  The running reference m of a row is
+		// only raised when some row of the wave exceeds it by more than kRescaleSlack
+		// (log2 units): until then P = exp2(x - m) may grow to 2^slack, which fp32 sums and
+		// 16-bit P hold without loss, and the O accumulators are left alone.
 		V8 pf[QB][BN / 16];
 #pragma unroll
 		for (int qb = 0; qb < QB; ++qb) {
@@ -247,12 +280,9 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const KArgs a) {
 			for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
 				for (int i = 0; i < 16; ++i) {
-					float x;
-					if constexpr (BIAS)
-						x = __builtin_fmaf(s[kb][qb][i], c1, bv[kb][qb][i >> 2][i & 3]);
-					else
-						x = s[kb][qb][i] * c1;
-					if (need_mask) {
+					float x = s[kb][qb][i];
+					if constexpr (BIAS) x = __builtin_fmaf(x, c1, bv[kb][qb][i >> 2][i & 3]);
+					if constexpr (MASKED) {
 						int j = n0 + 32 * kb + 8 * (i >> 2) + 4 * g + (i & 3);
 						x = j <= jmax[qb] ? x : -INFINITY;
 					}
@@ -260,20 +290,33 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const KArgs a) {
 					mx = __builtin_fmaxf(mx, x);
 				}
 			mx = pair_max(mx);
-			float m_new = __builtin_fmaxf(mrow[qb], mx);
-			float m_use = m_new == -INFINITY ? 0.f : m_new;
-			float alpha = BIAS ? exp2_fast((mrow[qb] - m_use) * kLog2e) : exp2_fast(mrow[qb] - m_use);
-			mrow[qb] = m_new;
+			// to the softmax domain (log2 units without bias, natural units with bias)
+			if constexpr (!BIAS) mx = mx * c1;  // c1 > 0 is checked by the launcher
+			const float slack = BIAS ? kRescaleSlack * kLn2 : kRescaleSlack;
+			if (__builtin_amdgcn_ballot_w64(mx > mrow[qb] + slack) != 0) {
+				float m_new = __builtin_fmaxf(mrow[qb], mx);
+				float m_use = m_new == -INFINITY ? 0.f : m_new;
+				float alpha = BIAS ? exp2_fast((mrow[qb] - m_use) * kLog2e) : exp2_fast(mrow[qb] - m_use);
+				mrow[qb] = m_new;
+				lrow[qb] *= alpha;
+#pragma unroll
+				for (int db = 0; db < DB; ++db)
+#pragma unroll
+					for (int i = 0; i < 16; ++i) oacc[qb][db][i] *= alpha;
+			}
+			const float m_use = mrow[qb] == -INFINITY ? 0.f : mrow[qb];
+			const float nm = BIAS ? -m_use * kLog2e : -m_use;
 			float lsum = 0.f;
 #pragma unroll
 			for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
 				for (int i = 0; i < 16; ++i) {
-					float p = BIAS ? exp2_fast((s[kb][qb][i] - m_use) * kLog2e) : exp2_fast(s[kb][qb][i] - m_use);
+					float p = BIAS ? exp2_fast(__builtin_fmaf(s[kb][qb][i] - m_use, kLog2e, 0.f))
+					               : exp2_fast(__builtin_fmaf(s[kb][qb][i], c1, nm));
 					lsum += p;
 					s[kb][qb][i] = p;
 				}
-			lrow[qb] = lrow[qb] * alpha + lsum;
+			lrow[qb] += lsum;
 			if constexpr (DROP) {
 #pragma unroll
 				for (int kb = 0; kb < KB; ++kb)
@@ -287,10 +330,6 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const KArgs a) {
 					}
 			}
 #pragma unroll
-			for (int db = 0; db < DB; ++db)
-#pragma unroll
-				for (int i = 0; i < 16; ++i) oacc[qb][db][i] *= alpha;
-#pragma unroll
 			for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
 				for (int hf = 0; hf < 2; ++hf) {
@@ -301,14 +340,43 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const KArgs a) {
 		}
 
 		// O^T += V^T P^T
+		auto pv_batch = [&](auto batch_tag) {
+			constexpr int BI = decltype(batch_tag)::value;
+			lds_tr_wait(vfr[BI & 1]);
+			if constexpr (BI + 1 < NBATCH) issue_v(std::integral_constant<int, BI + 1>{}, vfr[(BI + 1) & 1]);
 #pragma unroll
-		for (int kk = 0; kk < BN / 16; ++kk)
+			for (int f = 0; f < FPB; ++f)
 #pragma unroll
-			for (int db = 0; db < DB; ++db) {
-				V8 vf = lds_frag_tr<T, D>(vt, 16 * kk, 32 * db, lane);
+				for (int db = 0; db < DB; ++db)
 #pragma unroll
-				for (int qb = 0; qb < QB; ++qb) oacc[qb][db] = mfma32(vf, pf[qb][kk], oacc[qb][db]);
-			}
+					for (int qb = 0; qb < QB; ++qb)
+						oacc[qb][db] = mfma32(as_frag<T>(vfr[BI & 1][f * DB + db]), pf[qb][BI * FPB + f], oacc[qb][db]);
+		};
+		pv_batch(std::integral_constant<int, 0>{});
+		if constexpr (NBATCH > 1) pv_batch(std::integral_constant<int, 1>{});
+		if constexpr (NBATCH > 2) pv_batch(std::integral_constant<int, 2>{});
+		if constexpr (NBATCH > 3) pv_batch(std::integral_constant<int, 3>{});
+		static_assert(NBATCH <= 4, "");
+	};
+
+	for (int t = 0; t < ntiles; ++t) {
+		const int n0 = t * BN;
+		const int buf = t & 1;
+		wait_async_loads();
+		__syncthreads();
+		if (t + 1 < ntiles) {
+			int n1 = n0 + BN;
+			int rows = sk_eff - n1 < BN ? sk_eff - n1 : BN;
+			tile_load_async<D, BN, NT>(lds + (buf ^ 1) * TILE_BYTES, kbase + (int64_t)n1 * a.k.ss, a.k.ss, rows, tid);
+			tile_load_async<D, BN, NT>(lds + (2 + (buf ^ 1)) * TILE_BYTES, vbase + (int64_t)n1 * a.v.ss, a.v.ss, rows, tid);
+		}
+		if (n0 > wave_jmax) continue;  // whole tile masked for this wave (uniform)
+		const FA2_LDS char* kt = lds + buf * TILE_BYTES;
+		const FA2_LDS char* vt = lds + (2 + buf) * TILE_BYTES;
+		if (n0 + BN - 1 > wave_jmin)
+			tile_body(std::true_type{}, kt, vt, n0);
+		else
+			tile_body(std::false_type{}, kt, vt, n0);
 	}
 
 	// epilogue: normalise, store O (lane: row c, four consecutive d per store) and LSE
@@ -344,8 +412,8 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const KArgs a) {
 
 template <typename T, int D>
 struct FwdCfg {
-	static constexpr int NW = 4;
-	static constexpr int QB = D <= 128 ? 2 : 1;
+	static constexpr int NW = D <= 128 ? 8 : 4;
+	static constexpr int QB = 1;
 	static constexpr int BM = NW * QB * 32;
 };
 
