@@ -139,14 +139,14 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 
 	const float c1 = BIAS ? a.scale : a.scale * kLog2e;
 
-	auto issue_tile = [&](int step, int buf) {
+	auto issue_tile = [&](int step, FA2_LDS char* qdst, FA2_LDS char* dodst) {
 		int hq = hk * r + step / nq;
 		int m0 = (q_lo + step % nq) * BMQ;
 		int rows = a.Sq - m0 < BMQ ? a.Sq - m0 : BMQ;
 		const char* qb_ = a.q.ptr + (int64_t)b * a.q.sb + (int64_t)hq * a.q.sh + (int64_t)m0 * a.q.ss;
 		const char* db_ = a.dout.ptr + (int64_t)b * a.dout.sb + (int64_t)hq * a.dout.sh + (int64_t)m0 * a.dout.ss;
-		tile_load_async<D, BMQ, NT>(lds + buf * TILE_BYTES, qb_, a.q.ss, rows, tid);
-		tile_load_async<D, BMQ, NT>(lds + (2 + buf) * TILE_BYTES, db_, a.dout.ss, rows, tid);
+		tile_load_async<D, BMQ, NT>(qdst, qb_, a.q.ss, rows, tid);
+		tile_load_async<D, BMQ, NT>(dodst, db_, a.dout.ss, rows, tid);
 	};
 	// per-row statistics of a tile: thread t < BMQ fetches lse, t in [BMQ, 2 BMQ) fetches delta
 	auto fetch_stat = [&](int step) -> float {
@@ -192,10 +192,8 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 
 	// One streamed tile of BMQ query rows of q-head hq.  MASKED = some (row, key)
 	// of this wave's 32 keys x BMQ rows is masked.
-	auto tile_body = [&](auto masked_tag, int buf, int hq, int m0) {
+	auto tile_body = [&](auto masked_tag, const FA2_LDS char* qt, const FA2_LDS char* dot, int buf, int hq, int m0) {
 		constexpr bool MASKED = decltype(masked_tag)::value;
-		const FA2_LDS char* qt = lds + buf * TILE_BYTES;
-		const FA2_LDS char* dot = lds + (2 + buf) * TILE_BYTES;
 		const FA2_LDS char* lse_s = stat + buf * STAT_BYTES;
 		const FA2_LDS char* del_s = stat + (2 + buf) * STAT_BYTES;
 		const char* bias_base = nullptr;
@@ -205,9 +203,42 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 			int es = a.bias_dtype == 3 ? 4 : 2;
 			bias_base = a.bias + (int64_t)b * a.bias_sb + (int64_t)hb * a.bias_sh + (int64_t)jc * es;
 		}
-#pragma unroll 1
-		for (int qb = 0; qb < QB; ++qb) {
-			// bias column for this lane's key, 16 rows
+		// The tile's QB blocks of 32 rows go through three stages,
+		//   A(i): S_i = Q_i K^T, dP_i = dO_i V^T          (matrix products)
+		//   B(i): P_i, dS_i from S_i, dP_i, lse, delta      (elementwise)
+		//   C(i): dV^T += dO_i^T P_i, dK^T += Q_i^T dS_i   (matrix products)
+		// software-pipelined so that B(i) runs between the independent products
+		// A(i+1) and C(i-1): the elementwise math hides behind the matrix pipe.
+		constexpr int NFR = 2 * DB;  // transposed fragments of one 16-row half of a block: (dO^T, Q^T) x DB
+		f32x16 s[2], dp[2];
+		V8 pb[2][2], sb[2][2];
+		u32x4 tfr[2][NFR];  // [half]
+
+		auto stage_A = [&](int qb, f32x16& sa, f32x16& dpa) {
+#pragma unroll
+			for (int i = 0; i < 16; ++i) sa[i] = dpa[i] = 0.f;
+#pragma unroll
+			for (int ks = 0; ks < KS; ++ks) {
+				V8 qa = *(const FA2_LDS V8*)(qt + poff[ks] + qb * (32 * D * 2));
+				sa = mfma32(qa, kf[ks], sa);
+			}
+#pragma unroll
+			for (int ks = 0; ks < KS; ++ks) {
+				V8 da = *(const FA2_LDS V8*)(dot + poff[ks] + qb * (32 * D * 2));
+				dpa = mfma32(da, vf[ks], dpa);
+			}
+		};
+		// fragments of half `hf` of block qb
+		auto issue_C = [&](int qb, int hf, u32x4(&dst)[NFR]) {
+			const FA2_LDS char* dot_a = dot + qb * (32 * D * 2);
+			const FA2_LDS char* qt_a = qt + qb * (32 * D * 2);
+#pragma unroll
+			for (int db = 0; db < DB; ++db) {
+				dst[db] = lds_tr_issue_rt<D>(dot_a + toff[db][0], dot_a + toff[db][1], hf);
+				dst[DB + db] = lds_tr_issue_rt<D>(qt_a + toff[db][0], qt_a + toff[db][1], hf);
+			}
+		};
+		auto stage_B = [&](int qb, f32x16& sa, f32x16& dpa, V8(&pbo)[2], V8(&sbo)[2]) {
 			float bv[BIAS ? 16 : 1];
 			if constexpr (BIAS) {
 #pragma unroll
@@ -220,57 +251,27 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 					                            : (float)*(const _Float16*)pp;
 				}
 			}
-			f32x16 s, dp;
-#pragma unroll
-			for (int i = 0; i < 16; ++i) s[i] = dp[i] = 0.f;
-#pragma unroll
-			for (int ks = 0; ks < KS; ++ks) {
-				V8 qa = *(const FA2_LDS V8*)(qt + poff[ks] + qb * (32 * D * 2));
-				s = mfma32(qa, kf[ks], s);
-			}
-#pragma unroll
-			for (int ks = 0; ks < KS; ++ks) {
-				V8 da = *(const FA2_LDS V8*)(dot + poff[ks] + qb * (32 * D * 2));
-				dp = mfma32(da, vf[ks], dp);
-			}
-			// transposed fragments for the two products below, one batch per 16-row half:
-			// issued early so that their LDS latency is covered by the products above and
-			// by the elementwise math
-			constexpr bool BOTH_EARLY = DB <= 4;
-			u32x4 tfr[2][2 * DB];
-			const uint32_t dot_a = lds_addr(dot) + qb * (32 * D * 2);
-			const uint32_t qt_a = lds_addr(qt) + qb * (32 * D * 2);
-			auto issue_t = [&](int hf, u32x4(&dst)[2 * DB]) {
-#pragma unroll
-				for (int db = 0; db < DB; ++db) {
-					dst[2 * db] = lds_tr_issue_rt<D>(dot_a + toff[db][0], dot_a + toff[db][1], hf);
-					dst[2 * db + 1] = lds_tr_issue_rt<D>(qt_a + toff[db][0], qt_a + toff[db][1], hf);
-				}
-			};
-			issue_t(0, tfr[0]);
-			if constexpr (BOTH_EARLY) issue_t(1, tfr[1]);
 			f32x4 lse4[4], del4[4];
 #pragma unroll
 			for (int aa = 0; aa < 4; ++aa) {
 				lse4[aa] = *(const FA2_LDS f32x4*)(lse_s + (32 * qb + 8 * aa + 4 * g) * 4);
 				del4[aa] = *(const FA2_LDS f32x4*)(del_s + (32 * qb + 8 * aa + 4 * g) * 4);
 			}
-			__builtin_amdgcn_sched_barrier(0);
-			f32x16 pd;  // P after dropout (feeds dV); s becomes dS (feeds dK)
+			f32x16 pd;  // P after dropout (feeds dV); sa becomes dS (feeds dK)
 #pragma unroll
 			for (int i = 0; i < 16; ++i) {
 				int row = m0 + 32 * qb + 8 * (i >> 2) + 4 * g + (i & 3);
 				float lse = lse4[i >> 2][i & 3], del = del4[i >> 2][i & 3];
 				float p;
 				if constexpr (BIAS)
-					p = exp2_fast((__builtin_fmaf(s[i], c1, bv[i]) - lse) * kLog2e);
+					p = exp2_fast((__builtin_fmaf(sa[i], c1, bv[i]) - lse) * kLog2e);
 				else
-					p = exp2_fast(__builtin_fmaf(s[i], c1, -lse));
+					p = exp2_fast(__builtin_fmaf(sa[i], c1, -lse));
 				if constexpr (MASKED) {
 					bool ok = row < sq_eff && jcol < sk_eff && (!a.causal || jcol <= row + off);
 					p = ok ? p : 0.f;
 				}
-				float pdrop = p, dpe = dp[i];
+				float pdrop = p, dpe = dpa[i];
 				if constexpr (DROP) {
 					u32x4 rnd = philox4x32_10((uint32_t)(jcol >> 2), (uint32_t)row, (uint32_t)hq, (uint32_t)b, a.drop_k0, a.drop_k1);
 					uint32_t word = rnd[0];
@@ -282,59 +283,92 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 					dpe = keep ? dpe * a.drop_inv_keep : 0.f;
 				}
 				pd[i] = pdrop;
-				s[i] = p * (dpe - del);
+				sa[i] = p * (dpe - del);
 			}
-			// dV^T += dO^T P ; dK^T += Q^T dS   (k runs over the tile's 32 rows, two steps of 16)
 #pragma unroll
 			for (int hf = 0; hf < 2; ++hf) {
-				V8 pb = pack8<T>(pd[8 * hf + 0], pd[8 * hf + 1], pd[8 * hf + 2], pd[8 * hf + 3], pd[8 * hf + 4], pd[8 * hf + 5],
-				                 pd[8 * hf + 6], pd[8 * hf + 7]);
-				V8 sb = pack8<T>(s[8 * hf + 0], s[8 * hf + 1], s[8 * hf + 2], s[8 * hf + 3], s[8 * hf + 4], s[8 * hf + 5],
-				                 s[8 * hf + 6], s[8 * hf + 7]);
-				if (hf == 0 || !BOTH_EARLY) lds_tr_wait(tfr[hf]);
-				if (hf == 0 && !BOTH_EARLY) issue_t(1, tfr[1]);
+				pbo[hf] = pack8<T>(pd[8 * hf + 0], pd[8 * hf + 1], pd[8 * hf + 2], pd[8 * hf + 3], pd[8 * hf + 4], pd[8 * hf + 5],
+				                   pd[8 * hf + 6], pd[8 * hf + 7]);
+				sbo[hf] = pack8<T>(sa[8 * hf + 0], sa[8 * hf + 1], sa[8 * hf + 2], sa[8 * hf + 3], sa[8 * hf + 4], sa[8 * hf + 5],
+				                   sa[8 * hf + 6], sa[8 * hf + 7]);
+			}
+		};
+		// half 0's fragments were issued one stage earlier; half 1's are issued here and
+		// arrive while half 0's products run
+		auto stage_C = [&](int qb, V8(&pbi)[2], V8(&sbi)[2]) {
+			issue_C(qb, 1, tfr[1]);
+#pragma unroll
+			for (int hf = 0; hf < 2; ++hf)
 #pragma unroll
 				for (int db = 0; db < DB; ++db) {
-					dv[db] = mfma32(as_frag<T>(tfr[hf][2 * db]), pb, dv[db]);
-					dk[db] = mfma32(as_frag<T>(tfr[hf][2 * db + 1]), sb, dk[db]);
+					dv[db] = mfma32(as_frag<T>(tfr[hf][db]), pbi[hf], dv[db]);
+					dk[db] = mfma32(as_frag<T>(tfr[hf][DB + db]), sbi[hf], dk[db]);
 				}
+		};
+
+		stage_A(0, s[0], dp[0]);
+#pragma unroll
+		for (int k = 1; k <= QB + 1; ++k) {
+			if (k >= 2) stage_C(k - 2, pb[k & 1], sb[k & 1]);
+			if (k < QB) stage_A(k, s[k & 1], dp[k & 1]);
+			if (k - 1 < QB) {
+				issue_C(k - 1, 0, tfr[0]);
+				stage_B(k - 1, s[(k - 1) & 1], dp[(k - 1) & 1], pb[(k - 1) & 1], sb[(k - 1) & 1]);
 			}
 		}
 	};
 
 	if (steps > 0) {
-		issue_tile(0, 0);
+		issue_tile(0, lds, lds + 2 * TILE_BYTES);
 		store_stat(fetch_stat(0), 0);
 	}
 
-	for (int step = 0; step < steps; ++step) {
+	// One pipeline step: publish streamed tile `step`, start the copies of the next, compute.
+	auto run_step = [&](auto masked_tag, int step) {
 		const int buf = step & 1;
 		wait_async_loads();
 		__syncthreads();
 		float next_stat = 0.f;
 		const bool has_next = step + 1 < steps;
-		if (has_next) {
-#ifndef FA2_DBG_NOLOAD
-			issue_tile(step + 1, buf ^ 1);
-#endif
-			next_stat = fetch_stat(step + 1);
-		}
-		const int hq = hk * r + step / nq;
-		const int m0 = (q_lo + step % nq) * BMQ;
-		// wave-uniform: any work / any masking for (rows m0.., keys wn0..)?
-		int last_row = m0 + BMQ - 1 < sq_eff - 1 ? m0 + BMQ - 1 : sq_eff - 1;
-		bool skip = wn0 >= sk_eff || (a.causal && wn0 > last_row + off);
-#ifdef FA2_DBG_NOCOMPUTE
-		skip = true;
-#endif
-		if (!skip) {
-			const bool need_mask = (m0 + BMQ > sq_eff) || (wn0 + 32 > sk_eff) || (a.causal && wn0 + 31 > m0 + off);
-			if (need_mask)
-				tile_body(std::true_type{}, buf, hq, m0);
-			else
-				tile_body(std::false_type{}, buf, hq, m0);
-		}
+		lds_pipeline_step(
+		    lds + buf * TILE_BYTES, lds + (2 + buf) * TILE_BYTES, lds + (buf ^ 1) * TILE_BYTES, lds + (2 + (buf ^ 1)) * TILE_BYTES,
+		    [&](FA2_LDS char* nq_, FA2_LDS char* ndo) {
+			    if (has_next) {
+				    issue_tile(step + 1, nq_, ndo);
+				    next_stat = fetch_stat(step + 1);
+			    }
+		    },
+		    [&](const FA2_LDS char* qt, const FA2_LDS char* dot) {
+			    const int hq = hk * r + step / nq;
+			    const int m0 = (q_lo + step % nq) * BMQ;
+			    if constexpr (decltype(masked_tag)::value) {
+				    // wave-uniform: nothing to do for (rows m0.., keys wn0..)?
+				    int last_row = m0 + BMQ - 1 < sq_eff - 1 ? m0 + BMQ - 1 : sq_eff - 1;
+				    if (wn0 >= sk_eff || (a.causal && wn0 > last_row + off)) return;
+			    }
+			    tile_body(masked_tag, qt, dot, buf, hq, m0);
+		    });
 		if (has_next) store_stat(next_stat, buf ^ 1);
+	};
+	// Per q-head the streamed tiles are: tiles crossing this wave's causal diagonal
+	// (masked), tiles entirely below it (no mask), and a ragged last tile (masked).
+	// The unmasked tiles run in a loop of their own so that the steady state is a
+	// single straight-line body.
+	int i_diag = 0;  // first tile index (relative to q_lo) with no causal masking for this wave
+	if (a.causal) {
+		int first_clear = wn0 + 31 - off;  // rows >= this see all 32 keys of the wave
+		int tq = first_clear > 0 ? (first_clear + BMQ - 1) / BMQ : 0;
+		i_diag = tq - q_lo;
+	}
+	int i_full = sq_eff / BMQ - q_lo;  // tiles before this one lie entirely inside the valid rows
+	if (wn0 + 32 > sk_eff) i_diag = nq;  // ragged key block: always masked
+	i_diag = i_diag < 0 ? 0 : (i_diag > nq ? nq : i_diag);
+	i_full = i_full < i_diag ? i_diag : (i_full > nq ? nq : i_full);
+	for (int hi = 0; hi < r && nq > 0; ++hi) {
+		int base = hi * nq;
+		for (int i = 0; i < i_diag; ++i) run_step(std::true_type{}, base + i);
+		for (int i = i_diag; i < i_full; ++i) run_step(std::false_type{}, base + i);
+		for (int i = i_full; i < nq; ++i) run_step(std::true_type{}, base + i);
 	}
 
 	// epilogue: lane owns key jcol, four consecutive d per store
@@ -526,7 +560,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_kernel(const KArgs a) {
 			// K^T fragments for dQ^T += K^T dS^T, issued ahead of the elementwise math
 			constexpr bool BOTH_EARLY = DB <= 4;
 			u32x4 kfr[2][DB];
-			const uint32_t kt_a = lds_addr(kt) + kb * (32 * D * 2);
+			const FA2_LDS char* kt_a = kt + kb * (32 * D * 2);
 			auto issue_k = [&](int hf, u32x4(&dst)[DB]) {
 #pragma unroll
 				for (int db = 0; db < DB; ++db) dst[db] = lds_tr_issue_rt<D>(kt_a + toff[db][0], kt_a + toff[db][1], hf);
@@ -570,7 +604,6 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_kernel(const KArgs a) {
 			// dQ^T += K^T dS^T
 #pragma unroll
 			for (int hf = 0; hf < 2; ++hf) {
-				if (hf == 0 || !BOTH_EARLY) lds_tr_wait(kfr[hf]);
 				if (hf == 0 && !BOTH_EARLY) issue_k(1, kfr[1]);
 #pragma unroll
 				for (int db = 0; db < DB; ++db)
@@ -580,25 +613,36 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_kernel(const KArgs a) {
 		}
 	};
 
-	for (int t = 0; t < ntiles; ++t) {
+	// One pipeline step: publish tile t, start the copies of tile t + 1, compute.
+	auto step = [&](auto masked_tag, int t) {
 		const int n0 = t * BN;
 		const int buf = t & 1;
 		wait_async_loads();
 		__syncthreads();
-		if (t + 1 < ntiles) {
-			int n1 = n0 + BN;
-			int rows = sk_eff - n1 < BN ? sk_eff - n1 : BN;
-			tile_load_async<D, BN, NT>(lds + (buf ^ 1) * TILE_BYTES, kbase + (int64_t)n1 * a.k.ss, a.k.ss, rows, tid);
-			tile_load_async<D, BN, NT>(lds + (2 + (buf ^ 1)) * TILE_BYTES, vbase + (int64_t)n1 * a.v.ss, a.v.ss, rows, tid);
-		}
-		if (n0 > wave_jmax) continue;
-		const FA2_LDS char* kt = lds + buf * TILE_BYTES;
-		const FA2_LDS char* vt = lds + (2 + buf) * TILE_BYTES;
-		if (n0 + BN - 1 > wave_jmin)
-			tile_body(std::true_type{}, kt, vt, n0);
-		else
-			tile_body(std::false_type{}, kt, vt, n0);
-	}
+		lds_pipeline_step(
+		    lds + buf * TILE_BYTES, lds + (2 + buf) * TILE_BYTES, lds + (buf ^ 1) * TILE_BYTES, lds + (2 + (buf ^ 1)) * TILE_BYTES,
+		    [&](FA2_LDS char* nk, FA2_LDS char* nv) {
+			    if (t + 1 < ntiles) {
+				    int n1 = n0 + BN;
+				    int rows = sk_eff - n1 < BN ? sk_eff - n1 : BN;
+				    tile_load_async<D, BN, NT>(nk, kbase + (int64_t)n1 * a.k.ss, a.k.ss, rows, tid);
+				    tile_load_async<D, BN, NT>(nv, vbase + (int64_t)n1 * a.v.ss, a.v.ss, rows, tid);
+			    }
+		    },
+		    [&](const FA2_LDS char* kt, const FA2_LDS char* vt) {
+			    if constexpr (decltype(masked_tag)::value) {
+				    if (n0 > wave_jmax) return;  // whole tile masked for this wave (uniform)
+			    }
+			    tile_body(masked_tag, kt, vt, n0);
+		    });
+	};
+	// Tiles that lie entirely below every row's last allowed key need no mask.  They
+	// run in a loop of their own, so that the steady-state loop is a single
+	// straight-line body; the tiles on the causal diagonal / ragged end follow.
+	int t_full = (wave_jmin + 1) / BN;
+	t_full = t_full < 0 ? 0 : (t_full > ntiles ? ntiles : t_full);
+	for (int t = 0; t < t_full; ++t) step(std::false_type{}, t);
+	for (int t = t_full; t < ntiles; ++t) step(std::true_type{}, t);
 
 	char* obase = a.dq.ptr + (int64_t)b * a.dq.sb + (int64_t)h * a.dq.sh;
 #pragma unroll

@@ -131,63 +131,51 @@ FA2_DEV typename T::V8 lds_frag_tr(const FA2_LDS char* tile, int row0, int col0,
 	return __builtin_bit_cast(typename T::V8, both);
 }
 
-// Transposed fragments, issued and awaited separately.
-//
-// The direct global->LDS copies of the NEXT tile are in flight while the
-// current tile is read.  The compiler cannot tell that the two never overlap
-// and would put a full `s_waitcnt vmcnt(0)` in front of a transposed-read
-// intrinsic - which would serialise the double buffer.  So the transposed
-// reads are issued as inline asm (which the compiler does not treat as an LDS
-// access), and `lds_tr_wait` is the point where their results become usable:
-// it waits for all outstanding LDS reads and ties the fragment registers to
-// that wait so no use can be scheduled above it.  The workgroup barrier that
-// publishes a tile orders these reads against the copies that later overwrite it.
-//
-// IMM is a compile-time byte offset added to both addresses.
+// Transposed fragment from two per-lane byte addresses (rows r and r + 8) plus a
+// compile-time byte offset.  Returned as raw bits; as_frag<T>() views them as the
+// MFMA operand.
 template <int IMM>
-FA2_DEV u32x4 lds_tr_issue(uint32_t addr_lo, uint32_t addr_hi) {
-	u32x2 lo, hi;
-	asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(lo) : "v"(addr_lo), "n"(IMM));
-	asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(hi) : "v"(addr_hi), "n"(IMM));
-	u32x4 r = {lo.x, lo.y, hi.x, hi.y};
-	return r;
+FA2_DEV u32x4 lds_tr_issue(const FA2_LDS char* p_lo, const FA2_LDS char* p_hi) {
+	typedef __attribute__((__vector_size__(4 * sizeof(short)))) short v4s;
+	v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FA2_LDS v4s*)(p_lo + IMM));
+	v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FA2_LDS v4s*)(p_hi + IMM));
+	typedef __attribute__((__vector_size__(8 * sizeof(short)))) short v8s;
+	v8s both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+	return __builtin_bit_cast(u32x4, both);
 }
 
-// Same with the immediate chosen at run time among the 16-row steps 0..3 of a
-// tile with row length D (the loop index is a compile-time constant after
-// unrolling, so the switch folds away).
+// Same with the offset chosen among the 16-row steps 0..3 of a tile with row
+// length D (the step is a compile-time constant after unrolling, so the switch
+// folds away).
 template <int D>
-FA2_DEV u32x4 lds_tr_issue_rt(uint32_t addr_lo, uint32_t addr_hi, int step16) {
+FA2_DEV u32x4 lds_tr_issue_rt(const FA2_LDS char* p_lo, const FA2_LDS char* p_hi, int step16) {
 	switch (step16) {
-		case 0: return lds_tr_issue<0>(addr_lo, addr_hi);
-		case 1: return lds_tr_issue<16 * D * 2>(addr_lo, addr_hi);
-		case 2: return lds_tr_issue<32 * D * 2>(addr_lo, addr_hi);
-		default: return lds_tr_issue<48 * D * 2>(addr_lo, addr_hi);
+		case 0: return lds_tr_issue<0>(p_lo, p_hi);
+		case 1: return lds_tr_issue<16 * D * 2>(p_lo, p_hi);
+		case 2: return lds_tr_issue<32 * D * 2>(p_lo, p_hi);
+		default: return lds_tr_issue<48 * D * 2>(p_lo, p_hi);
 	}
 }
 
-template <int N>
-FA2_DEV void lds_tr_wait(u32x4 (&f)[N]) {
-	static_assert(N == 2 || N == 4 || N == 8 || N == 16, "unsupported fragment count");
-	if constexpr (N == 2)
-		asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f[0]), "+v"(f[1]));
-	else if constexpr (N == 4)
-		asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]));
-	else if constexpr (N == 8)
-		asm volatile("s_waitcnt lgkmcnt(0)"
-		             : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]), "+v"(f[4]), "+v"(f[5]), "+v"(f[6]), "+v"(f[7]));
-	else
-		asm volatile("s_waitcnt lgkmcnt(0)"
-		             : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]), "+v"(f[4]), "+v"(f[5]), "+v"(f[6]), "+v"(f[7]),
-		               "+v"(f[8]), "+v"(f[9]), "+v"(f[10]), "+v"(f[11]), "+v"(f[12]), "+v"(f[13]), "+v"(f[14]), "+v"(f[15]));
+// One step of a double-buffered LDS pipeline.  `issue(next0, next1)` starts the
+// direct global->LDS copies of the next tile, `body(cur0, cur1)` computes on the
+// current one.  The four regions are distinct; declaring them __restrict__ here
+// is what lets the compiler see that the LDS reads of `body` never touch the
+// regions the copies are filling - without it every transposed read would be
+// preceded by a wait for ALL outstanding copies (s_waitcnt vmcnt(0)), which
+// would serialise the double buffer.
+template <typename Issue, typename Body>
+FA2_DEV void lds_pipeline_step(const FA2_LDS char* __restrict__ cur0, const FA2_LDS char* __restrict__ cur1,
+                               FA2_LDS char* __restrict__ next0, FA2_LDS char* __restrict__ next1, Issue&& issue,
+                               Body&& body) {
+	issue(next0, next1);
+	body(cur0, cur1);
 }
 
 template <typename T>
 FA2_DEV typename T::V8 as_frag(u32x4 x) {
 	return __builtin_bit_cast(typename T::V8, x);
 }
-
-FA2_DEV uint32_t lds_addr(const FA2_LDS char* p) { return (uint32_t)(uintptr_t)p; }
 
 // Copy a ROWS x D tile from global memory (row stride `stride` elements) into
 // a swizzled LDS tile without passing through registers.  Each wave-level

@@ -256,14 +256,13 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const KArgs a) {
 		constexpr int NBATCH = KK / FPB;
 		constexpr int NF = FPB * DB;
 		u32x4 vfr[2][NF];
-		const uint32_t vt_a = lds_addr(vt);
 		auto issue_v = [&](auto batch_tag, u32x4(&dst)[NF]) {
 			constexpr int BI = decltype(batch_tag)::value;
 #pragma unroll
 			for (int f = 0; f < FPB; ++f)
 #pragma unroll
 				for (int db = 0; db < DB; ++db) {
-					dst[f * DB + db] = lds_tr_issue_rt<D>(vt_a + voff[db][0], vt_a + voff[db][1], BI * FPB + f);
+					dst[f * DB + db] = lds_tr_issue_rt<D>(vt + voff[db][0], vt + voff[db][1], BI * FPB + f);
 				}
 		};
 		issue_v(std::integral_constant<int, 0>{}, vfr[0]);
@@ -342,7 +341,6 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const KArgs a) {
 		// O^T += V^T P^T
 		auto pv_batch = [&](auto batch_tag) {
 			constexpr int BI = decltype(batch_tag)::value;
-			lds_tr_wait(vfr[BI & 1]);
 			if constexpr (BI + 1 < NBATCH) issue_v(std::integral_constant<int, BI + 1>{}, vfr[(BI + 1) & 1]);
 #pragma unroll
 			for (int f = 0; f < FPB; ++f)
@@ -359,25 +357,36 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const KArgs a) {
 		static_assert(NBATCH <= 4, "");
 	};
 
-	for (int t = 0; t < ntiles; ++t) {
+	// One pipeline step: publish tile t, start the copies of tile t + 1, compute.
+	auto step = [&](auto masked_tag, int t) {
 		const int n0 = t * BN;
 		const int buf = t & 1;
 		wait_async_loads();
 		__syncthreads();
-		if (t + 1 < ntiles) {
-			int n1 = n0 + BN;
-			int rows = sk_eff - n1 < BN ? sk_eff - n1 : BN;
-			tile_load_async<D, BN, NT>(lds + (buf ^ 1) * TILE_BYTES, kbase + (int64_t)n1 * a.k.ss, a.k.ss, rows, tid);
-			tile_load_async<D, BN, NT>(lds + (2 + (buf ^ 1)) * TILE_BYTES, vbase + (int64_t)n1 * a.v.ss, a.v.ss, rows, tid);
-		}
-		if (n0 > wave_jmax) continue;  // whole tile masked for this wave (uniform)
-		const FA2_LDS char* kt = lds + buf * TILE_BYTES;
-		const FA2_LDS char* vt = lds + (2 + buf) * TILE_BYTES;
-		if (n0 + BN - 1 > wave_jmin)
-			tile_body(std::true_type{}, kt, vt, n0);
-		else
-			tile_body(std::false_type{}, kt, vt, n0);
-	}
+		lds_pipeline_step(
+		    lds + buf * TILE_BYTES, lds + (2 + buf) * TILE_BYTES, lds + (buf ^ 1) * TILE_BYTES, lds + (2 + (buf ^ 1)) * TILE_BYTES,
+		    [&](FA2_LDS char* nk, FA2_LDS char* nv) {
+			    if (t + 1 < ntiles) {
+				    int n1 = n0 + BN;
+				    int rows = sk_eff - n1 < BN ? sk_eff - n1 : BN;
+				    tile_load_async<D, BN, NT>(nk, kbase + (int64_t)n1 * a.k.ss, a.k.ss, rows, tid);
+				    tile_load_async<D, BN, NT>(nv, vbase + (int64_t)n1 * a.v.ss, a.v.ss, rows, tid);
+			    }
+		    },
+		    [&](const FA2_LDS char* kt, const FA2_LDS char* vt) {
+			    if constexpr (decltype(masked_tag)::value) {
+				    if (n0 > wave_jmax) return;  // whole tile masked for this wave (uniform)
+			    }
+			    tile_body(masked_tag, kt, vt, n0);
+		    });
+	};
+	// Tiles that lie entirely below every row's last allowed key need no mask.  They
+	// run in a loop of their own, so that the steady-state loop is a single
+	// straight-line body; the tiles on the causal diagonal / ragged end follow.
+	int t_full = (wave_jmin + 1) / BN;
+	t_full = t_full < 0 ? 0 : (t_full > ntiles ? ntiles : t_full);
+	for (int t = 0; t < t_full; ++t) step(std::false_type{}, t);
+	for (int t = t_full; t < ntiles; ++t) step(std::true_type{}, t);
 
 	// epilogue: normalise, store O (lane: row c, four consecutive d per store) and LSE
 	char* obase = a.o.ptr + (int64_t)b * a.o.sb + (int64_t)h * a.o.sh;
