@@ -204,42 +204,38 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 			bias_base = a.bias + (int64_t)b * a.bias_sb + (int64_t)hb * a.bias_sh + (int64_t)jc * es;
 		}
 		// The tile's QB blocks of 32 rows go through three stages,
-		//   A(i): S_i = Q_i K^T, dP_i = dO_i V^T          (matrix products)
-		//   B(i): P_i, dS_i from S_i, dP_i, lse, delta      (elementwise)
-		//   C(i): dV^T += dO_i^T P_i, dK^T += Q_i^T dS_i   (matrix products)
-		// software-pipelined so that B(i) runs between the independent products
-		// A(i+1) and C(i-1): the elementwise math hides behind the matrix pipe.
+		//   A(i): S_i = Q_i K^T, dP_i = dO_i V^T          (2 KS matrix products)
+		//   B(i): P_i, dS_i from S_i, dP_i, lse, delta      (elementwise, 16 values per lane)
+		//   C(i): dV^T += dO_i^T P_i, dK^T += Q_i^T dS_i   (4 DB matrix products)
+		// software-pipelined: pipeline stage k runs A(k), B(k-1) and C(k-2) together, cut
+		// into NCH chunks.  Chunk c issues its share of the products of A(k) and C(k-2),
+		// then the transposed LDS reads that feed later products, then the elementwise
+		// math of EPC of the 16 values of B(k-1) - so the vector ALU works in the shadow
+		// of the matrix pipe.  A scheduling barrier after every chunk pins that order.
 		constexpr int NFR = 2 * DB;  // transposed fragments of one 16-row half of a block: (dO^T, Q^T) x DB
+		constexpr int NCH = 8;            // chunks per stage
+		constexpr int EPC = 16 / NCH;     // elementwise values per chunk
 		f32x16 s[2], dp[2];
 		V8 pb[2][2], sb[2][2];
 		u32x4 tfr[2][NFR];  // [half]
+		V8 qa[KS], da[KS];
+		f32x4 lse4[4], del4[4];
+		f32x16 pd;  // P after dropout of the block in B (feeds dV); its S becomes dS (feeds dK)
+		float bv[BIAS ? 16 : 1];
 
-		auto stage_A = [&](int qb, f32x16& sa, f32x16& dpa) {
-#pragma unroll
-			for (int i = 0; i < 16; ++i) sa[i] = dpa[i] = 0.f;
+		auto load_A = [&](int qb) {
 #pragma unroll
 			for (int ks = 0; ks < KS; ++ks) {
-				V8 qa = *(const FA2_LDS V8*)(qt + poff[ks] + qb * (32 * D * 2));
-				sa = mfma32(qa, kf[ks], sa);
-			}
-#pragma unroll
-			for (int ks = 0; ks < KS; ++ks) {
-				V8 da = *(const FA2_LDS V8*)(dot + poff[ks] + qb * (32 * D * 2));
-				dpa = mfma32(da, vf[ks], dpa);
+				qa[ks] = *(const FA2_LDS V8*)(qt + poff[ks] + qb * (32 * D * 2));
+				da[ks] = *(const FA2_LDS V8*)(dot + poff[ks] + qb * (32 * D * 2));
 			}
 		};
-		// fragments of half `hf` of block qb
-		auto issue_C = [&](int qb, int hf, u32x4(&dst)[NFR]) {
-			const FA2_LDS char* dot_a = dot + qb * (32 * D * 2);
-			const FA2_LDS char* qt_a = qt + qb * (32 * D * 2);
+		auto load_stats = [&](int qb) {
 #pragma unroll
-			for (int db = 0; db < DB; ++db) {
-				dst[db] = lds_tr_issue_rt<D>(dot_a + toff[db][0], dot_a + toff[db][1], hf);
-				dst[DB + db] = lds_tr_issue_rt<D>(qt_a + toff[db][0], qt_a + toff[db][1], hf);
+			for (int aa = 0; aa < 4; ++aa) {
+				lse4[aa] = *(const FA2_LDS f32x4*)(lse_s + (32 * qb + 8 * aa + 4 * g) * 4);
+				del4[aa] = *(const FA2_LDS f32x4*)(del_s + (32 * qb + 8 * aa + 4 * g) * 4);
 			}
-		};
-		auto stage_B = [&](int qb, f32x16& sa, f32x16& dpa, V8(&pbo)[2], V8(&sbo)[2]) {
-			float bv[BIAS ? 16 : 1];
 			if constexpr (BIAS) {
 #pragma unroll
 				for (int i = 0; i < 16; ++i) {
@@ -251,71 +247,111 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 					                            : (float)*(const _Float16*)pp;
 				}
 			}
-			f32x4 lse4[4], del4[4];
-#pragma unroll
-			for (int aa = 0; aa < 4; ++aa) {
-				lse4[aa] = *(const FA2_LDS f32x4*)(lse_s + (32 * qb + 8 * aa + 4 * g) * 4);
-				del4[aa] = *(const FA2_LDS f32x4*)(del_s + (32 * qb + 8 * aa + 4 * g) * 4);
-			}
-			f32x16 pd;  // P after dropout (feeds dV); sa becomes dS (feeds dK)
-#pragma unroll
-			for (int i = 0; i < 16; ++i) {
-				int row = m0 + 32 * qb + 8 * (i >> 2) + 4 * g + (i & 3);
-				float lse = lse4[i >> 2][i & 3], del = del4[i >> 2][i & 3];
-				float p;
-				if constexpr (BIAS)
-					p = exp2_fast((__builtin_fmaf(sa[i], c1, bv[i]) - lse) * kLog2e);
-				else
-					p = exp2_fast(__builtin_fmaf(sa[i], c1, -lse));
-				if constexpr (MASKED) {
-					bool ok = row < sq_eff && jcol < sk_eff && (!a.causal || jcol <= row + off);
-					p = ok ? p : 0.f;
-				}
-				float pdrop = p, dpe = dpa[i];
-				if constexpr (DROP) {
-					u32x4 rnd = philox4x32_10((uint32_t)(jcol >> 2), (uint32_t)row, (uint32_t)hq, (uint32_t)b, a.drop_k0, a.drop_k1);
-					uint32_t word = rnd[0];
-					word = (jcol & 3) == 1 ? rnd[1] : word;
-					word = (jcol & 3) == 2 ? rnd[2] : word;
-					word = (jcol & 3) == 3 ? rnd[3] : word;
-					bool keep = word >= a.drop_thr;
-					pdrop = keep ? p : 0.f;
-					dpe = keep ? dpe * a.drop_inv_keep : 0.f;
-				}
-				pd[i] = pdrop;
-				sa[i] = p * (dpe - del);
-			}
-#pragma unroll
-			for (int hf = 0; hf < 2; ++hf) {
-				pbo[hf] = pack8<T>(pd[8 * hf + 0], pd[8 * hf + 1], pd[8 * hf + 2], pd[8 * hf + 3], pd[8 * hf + 4], pd[8 * hf + 5],
-				                   pd[8 * hf + 6], pd[8 * hf + 7]);
-				sbo[hf] = pack8<T>(sa[8 * hf + 0], sa[8 * hf + 1], sa[8 * hf + 2], sa[8 * hf + 3], sa[8 * hf + 4], sa[8 * hf + 5],
-				                   sa[8 * hf + 6], sa[8 * hf + 7]);
-			}
 		};
-		// half 0's fragments were issued one stage earlier; half 1's are issued here and
-		// arrive while half 0's products run
-		auto stage_C = [&](int qb, V8(&pbi)[2], V8(&sbi)[2]) {
-			issue_C(qb, 1, tfr[1]);
-#pragma unroll
-			for (int hf = 0; hf < 2; ++hf)
-#pragma unroll
-				for (int db = 0; db < DB; ++db) {
-					dv[db] = mfma32(as_frag<T>(tfr[hf][db]), pbi[hf], dv[db]);
-					dk[db] = mfma32(as_frag<T>(tfr[hf][DB + db]), sbi[hf], dk[db]);
-				}
+		// product j of A: even j -> S, odd j -> dP, k-step j / 2
+		auto mfma_A = [&](int j, f32x16& sa, f32x16& dpa) {
+			int ks = j >> 1;
+			if (j & 1)
+				dpa = mfma32(da[ks], vf[ks], dpa);
+			else
+				sa = mfma32(qa[ks], kf[ks], sa);
+		};
+		// product j of C: half j / (2 DB); inside a half even -> dV, odd -> dK, d-block (j % (2 DB)) / 2
+		auto mfma_C = [&](int j, V8(&pbi)[2], V8(&sbi)[2]) {
+			int hf = j / (2 * DB), rr = j % (2 * DB), db = rr >> 1;
+			if (rr & 1)
+				dk[db] = mfma32(as_frag<T>(tfr[hf][DB + db]), sbi[hf], dk[db]);
+			else
+				dv[db] = mfma32(as_frag<T>(tfr[hf][db]), pbi[hf], dv[db]);
+		};
+		// transposed fragment j of half hf of block qb: j < DB -> dO^T block j, else Q^T block j - DB
+		auto issue_tr = [&](int qb, int hf, int j, u32x4(&dst)[NFR]) {
+			const FA2_LDS char* base = (j < DB ? dot : qt) + qb * (32 * D * 2);
+			int db = j < DB ? j : j - DB;
+			dst[j] = lds_tr_issue_rt<D>(base + toff[db][0], base + toff[db][1], hf);
+		};
+		// value i of B(qb)
+		auto elem_B = [&](int qb, int i, f32x16& sa, f32x16& dpa) {
+			int row = m0 + 32 * qb + 8 * (i >> 2) + 4 * g + (i & 3);
+			float lse = lse4[i >> 2][i & 3], del = del4[i >> 2][i & 3];
+			float p;
+			if constexpr (BIAS)
+				p = exp2_fast((__builtin_fmaf(sa[i], c1, bv[i]) - lse) * kLog2e);
+			else
+				p = exp2_fast(__builtin_fmaf(sa[i], c1, -lse));
+			if constexpr (MASKED) {
+				bool ok = row < sq_eff && jcol < sk_eff && (!a.causal || jcol <= row + off);
+				p = ok ? p : 0.f;
+			}
+			float pdrop = p, dpe = dpa[i];
+			if constexpr (DROP) {
+				u32x4 rnd = philox4x32_10((uint32_t)(jcol >> 2), (uint32_t)row, (uint32_t)hq, (uint32_t)b, a.drop_k0, a.drop_k1);
+				uint32_t word = rnd[0];
+				word = (jcol & 3) == 1 ? rnd[1] : word;
+				word = (jcol & 3) == 2 ? rnd[2] : word;
+				word = (jcol & 3) == 3 ? rnd[3] : word;
+				bool keep = word >= a.drop_thr;
+				pdrop = keep ? p : 0.f;
+				dpe = keep ? dpe * a.drop_inv_keep : 0.f;
+			}
+			pd[i] = pdrop;
+			sa[i] = p * (dpe - del);
+		};
+		auto pack_B = [&](int hf, f32x16& sa, V8(&pbo)[2], V8(&sbo)[2]) {
+			pbo[hf] = pack8<T>(pd[8 * hf + 0], pd[8 * hf + 1], pd[8 * hf + 2], pd[8 * hf + 3], pd[8 * hf + 4], pd[8 * hf + 5],
+			                   pd[8 * hf + 6], pd[8 * hf + 7]);
+			sbo[hf] = pack8<T>(sa[8 * hf + 0], sa[8 * hf + 1], sa[8 * hf + 2], sa[8 * hf + 3], sa[8 * hf + 4], sa[8 * hf + 5],
+			                   sa[8 * hf + 6], sa[8 * hf + 7]);
 		};
 
-		stage_A(0, s[0], dp[0]);
+		auto stage = [&](auto k_tag) {
+			constexpr int k = decltype(k_tag)::value;
+			constexpr bool HAS_C = k >= 2, HAS_A = k < QB, HAS_B = k >= 1 && k - 1 < QB;
+			__builtin_amdgcn_sched_barrier(0);
+			if constexpr (HAS_B) load_stats(k - 1);
+			if constexpr (HAS_A) {
+				load_A(k);
 #pragma unroll
-		for (int k = 1; k <= QB + 1; ++k) {
-			if (k >= 2) stage_C(k - 2, pb[k & 1], sb[k & 1]);
-			if (k < QB) stage_A(k, s[k & 1], dp[k & 1]);
-			if (k - 1 < QB) {
-				issue_C(k - 1, 0, tfr[0]);
-				stage_B(k - 1, s[(k - 1) & 1], dp[(k - 1) & 1], pb[(k - 1) & 1], sb[(k - 1) & 1]);
+				for (int i = 0; i < 16; ++i) s[k & 1][i] = dp[k & 1][i] = 0.f;
 			}
-		}
+			__builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+			for (int c = 0; c < NCH; ++c) {
+				if constexpr (HAS_A) {
+#pragma unroll
+					for (int j = c * (2 * KS) / NCH; j < (c + 1) * (2 * KS) / NCH; ++j) mfma_A(j, s[k & 1], dp[k & 1]);
+				}
+				if constexpr (HAS_C) {
+#pragma unroll
+					for (int j = c * (4 * DB) / NCH; j < (c + 1) * (4 * DB) / NCH; ++j) mfma_C(j, pb[k & 1], sb[k & 1]);
+					// second half of C(k-2)'s fragments: read during the first eight chunks, used in the last eight
+					if (c < NCH / 2) {
+#pragma unroll
+						for (int j = c * NFR / (NCH / 2); j < (c + 1) * NFR / (NCH / 2); ++j) issue_tr(k - 2, 1, j, tfr[1]);
+					}
+				}
+				if constexpr (HAS_B) {
+					// first half of C(k-1)'s fragments, into the buffer C(k-2) has finished with
+					if (c >= NCH / 2) {
+#pragma unroll
+						for (int j = (c - NCH / 2) * NFR / (NCH / 2); j < (c - NCH / 2 + 1) * NFR / (NCH / 2); ++j)
+							issue_tr(k - 1, 0, j, tfr[0]);
+					}
+#pragma unroll
+					for (int e = 0; e < EPC; ++e) elem_B(k - 1, c * EPC + e, s[(k - 1) & 1], dp[(k - 1) & 1]);
+					if (c == NCH / 2 - 1) pack_B(0, s[(k - 1) & 1], pb[(k - 1) & 1], sb[(k - 1) & 1]);
+					if (c == NCH - 1) pack_B(1, s[(k - 1) & 1], pb[(k - 1) & 1], sb[(k - 1) & 1]);
+				}
+				__builtin_amdgcn_sched_barrier(0);
+			}
+		};
+		stage(std::integral_constant<int, 0>{});
+		stage(std::integral_constant<int, 1>{});
+		stage(std::integral_constant<int, 2>{});
+		if constexpr (QB + 1 >= 3) stage(std::integral_constant<int, 3>{});
+		if constexpr (QB + 1 >= 4) stage(std::integral_constant<int, 4>{});
+		if constexpr (QB + 1 >= 5) stage(std::integral_constant<int, 5>{});
+		static_assert(QB <= 4, "");
 	};
 
 	if (steps > 0) {
@@ -334,8 +370,10 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		    lds + buf * TILE_BYTES, lds + (2 + buf) * TILE_BYTES, lds + (buf ^ 1) * TILE_BYTES, lds + (2 + (buf ^ 1)) * TILE_BYTES,
 		    [&](FA2_LDS char* nq_, FA2_LDS char* ndo) {
 			    if (has_next) {
-				    issue_tile(step + 1, nq_, ndo);
+				    // statistics first: loads return in order, so waiting for this small load later
+				    // does not wait for the tile copies issued after it
 				    next_stat = fetch_stat(step + 1);
+				    issue_tile(step + 1, nq_, ndo);
 			    }
 		    },
 		    [&](const FA2_LDS char* qt, const FA2_LDS char* dot) {
@@ -668,7 +706,7 @@ template <typename T, int D>
 struct BwdCfg {
 	// dK/dV: 4 waves x 32 keys; query rows streamed 64 (32 for D = 256) at a time
 	static constexpr int KV_NW = 4;
-	static constexpr int KV_QB = D <= 128 ? 2 : 1;
+	static constexpr int KV_QB = D <= 128 ? 4 : 1;
 	static constexpr int KV_BN = KV_NW * 32;
 	// dQ: 4 waves x QB x 32 rows
 	static constexpr int DQ_NW = D <= 128 ? 8 : 4;
