@@ -1,0 +1,177 @@
+// XLA FFI handlers: the JAX-side entry into libfa2_hip.so.
+//
+// Each handler only translates XLA buffers and attributes into an fa2_params
+// block and calls the plain C ABI (fa2_fwd / fa2_bwd / fa2_dropout_mask,
+// include/fa2.h) on the stream XLA hands over.  They take the place of the
+// custom calls the reference emits through eformer.callib.triton_call
+// (jax_flash_attn2/flash_attention_triton/_forward_triton.py:547-588,
+//  _backward_triton.py:1049-1154).
+//
+// This file needs the XLA FFI headers that ship inside jaxlib
+// (`jax.ffi.include_dir()`); it is compiled into libfa2_xla_ffi.so by
+// `make ffi XLA_FFI_INCLUDE=<dir>` and is not part of the default build.
+//
+// Operand convention (absent optional operands are passed as 0-element buffers):
+//   fa2_fwd_ffi : args q, k, v, bias, seqlens        rets o, lse
+//   fa2_bwd_ffi : args q, k, v, bias, seqlens, o, lse, dout   rets dq, dk, dv, scratch
+//   attrs (both): scale f32, dropout_p f32, causal bool, seed i64, bias_group bool
+// All tensors are dense row-major as XLA lays them out: q/o/dout/dq [B,Sq,Hq,D],
+// k/v/dk/dv [B,Sk,Hkv,D], bias [B|1, H|1, Sq, Sk], lse [B,Hq,Sq] f32,
+// scratch [fa2_bwd_scratch_bytes] u8.
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+
+#include "../../include/fa2.h"
+#include "xla/ffi/api/ffi.h"
+
+namespace ffi = xla::ffi;
+
+namespace {
+
+int elem_type(ffi::DataType t) {
+	switch (t) {
+		case ffi::DataType::F16: return FA2_FP16;
+		case ffi::DataType::BF16: return FA2_BF16;
+		case ffi::DataType::F32: return FA2_FP32;
+		default: return 0;
+	}
+}
+
+fa2_tensor dense4(void* ptr, ffi::Span<const int64_t> d) {
+	fa2_tensor t;
+	t.ptr = ptr;
+	t.stride_b = d[1] * d[2] * d[3];
+	t.stride_s = d[2] * d[3];
+	t.stride_h = d[3];
+	return t;
+}
+
+ffi::Error fill_common(fa2_params& p, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::AnyBuffer v, ffi::AnyBuffer bias,
+                       ffi::AnyBuffer seqlens, float scale, float dropout_p, bool causal, int64_t seed, bool bias_group) {
+	std::memset(&p, 0, sizeof(p));
+	p.struct_size = sizeof(p);
+	auto qd = q.dimensions(), kd = k.dimensions();
+	if (qd.size() != 4 || kd.size() != 4 || v.dimensions().size() != 4)
+		return ffi::Error(ffi::ErrorCode::kInvalidArgument, "q, k, v must be [B, S, H, D]");
+	p.dtype = elem_type(q.element_type());
+	p.B = (int32_t)qd[0];
+	p.Sq = (int32_t)qd[1];
+	p.Hq = (int32_t)qd[2];
+	p.D = (int32_t)qd[3];
+	p.Sk = (int32_t)kd[1];
+	p.Hkv = (int32_t)kd[2];
+	p.causal = causal ? 1 : 0;
+	p.scale = scale;
+	p.p_drop = dropout_p;
+	p.seed = (uint64_t)seed;
+	p.q = dense4(q.untyped_data(), qd);
+	p.k = dense4(k.untyped_data(), kd);
+	p.v = dense4(v.untyped_data(), v.dimensions());
+	if (bias.element_count() > 0) {
+		auto bd = bias.dimensions();
+		if (bd.size() != 4) return ffi::Error(ffi::ErrorCode::kInvalidArgument, "bias must be 4-D");
+		p.bias = bias.untyped_data();
+		p.bias_dtype = elem_type(bias.element_type());
+		p.bias_stride_m = bd[3];
+		p.bias_stride_h = bd[1] == 1 ? 0 : bd[2] * bd[3];
+		p.bias_stride_b = bd[0] == 1 ? 0 : bd[1] * bd[2] * bd[3];
+		p.bias_group = bias_group ? 1 : 0;
+	}
+	if (seqlens.element_count() > 0) p.seqlens = (const int32_t*)seqlens.untyped_data();
+	return ffi::Error::Success();
+}
+
+ffi::Error to_error(int rc) {
+	if (rc == FA2_OK) return ffi::Error::Success();
+	return ffi::Error(rc == FA2_EHIP ? ffi::ErrorCode::kInternal : ffi::ErrorCode::kInvalidArgument, fa2_strerror(rc));
+}
+
+ffi::Error FwdImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::AnyBuffer v, ffi::AnyBuffer bias,
+                   ffi::AnyBuffer seqlens, ffi::Result<ffi::AnyBuffer> o, ffi::Result<ffi::AnyBuffer> lse, float scale,
+                   float dropout_p, bool causal, int64_t seed, bool bias_group) {
+	fa2_params p;
+	if (auto e = fill_common(p, q, k, v, bias, seqlens, scale, dropout_p, causal, seed, bias_group); e.failure()) return e;
+	p.o = dense4(o->untyped_data(), q.dimensions());
+	p.lse = (float*)lse->untyped_data();
+	return to_error(fa2_fwd(&p, stream));
+}
+
+ffi::Error BwdImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::AnyBuffer v, ffi::AnyBuffer bias,
+                   ffi::AnyBuffer seqlens, ffi::AnyBuffer o, ffi::AnyBuffer lse, ffi::AnyBuffer dout,
+                   ffi::Result<ffi::AnyBuffer> dq, ffi::Result<ffi::AnyBuffer> dk, ffi::Result<ffi::AnyBuffer> dv,
+                   ffi::Result<ffi::AnyBuffer> scratch, float scale, float dropout_p, bool causal, int64_t seed,
+                   bool bias_group) {
+	fa2_params p;
+	if (auto e = fill_common(p, q, k, v, bias, seqlens, scale, dropout_p, causal, seed, bias_group); e.failure()) return e;
+	p.o = dense4(o.untyped_data(), q.dimensions());
+	p.lse = (float*)lse.untyped_data();
+	p.dout = dense4(dout.untyped_data(), q.dimensions());
+	p.dq = dense4(dq->untyped_data(), q.dimensions());
+	p.dk = dense4(dk->untyped_data(), k.dimensions());
+	p.dv = dense4(dv->untyped_data(), v.dimensions());
+	p.scratch = scratch->untyped_data();
+	p.scratch_bytes = scratch->size_bytes();
+	return to_error(fa2_bwd(&p, stream));
+}
+
+ffi::Error DropoutMaskImpl(hipStream_t stream, ffi::Result<ffi::AnyBuffer> keep, float dropout_p, int64_t seed) {
+	auto d = keep->dimensions();  // [B, H, Sq, Sk] u8
+	if (d.size() != 4) return ffi::Error(ffi::ErrorCode::kInvalidArgument, "keep must be [B, H, Sq, Sk]");
+	fa2_params p;
+	std::memset(&p, 0, sizeof(p));
+	p.struct_size = sizeof(p);
+	p.B = (int32_t)d[0];
+	p.Hq = p.Hkv = (int32_t)d[1];
+	p.Sq = (int32_t)d[2];
+	p.Sk = (int32_t)d[3];
+	p.p_drop = dropout_p;
+	p.seed = (uint64_t)seed;
+	return to_error(fa2_dropout_mask(&p, (uint8_t*)keep->untyped_data(), stream));
+}
+
+}  // namespace
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(fa2_fwd_ffi, FwdImpl,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::AnyBuffer>()  // q
+                                  .Arg<ffi::AnyBuffer>()  // k
+                                  .Arg<ffi::AnyBuffer>()  // v
+                                  .Arg<ffi::AnyBuffer>()  // bias
+                                  .Arg<ffi::AnyBuffer>()  // seqlens
+                                  .Ret<ffi::AnyBuffer>()  // o
+                                  .Ret<ffi::AnyBuffer>()  // lse
+                                  .Attr<float>("scale")
+                                  .Attr<float>("dropout_p")
+                                  .Attr<bool>("causal")
+                                  .Attr<int64_t>("seed")
+                                  .Attr<bool>("bias_group"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(fa2_bwd_ffi, BwdImpl,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::AnyBuffer>()  // q
+                                  .Arg<ffi::AnyBuffer>()  // k
+                                  .Arg<ffi::AnyBuffer>()  // v
+                                  .Arg<ffi::AnyBuffer>()  // bias
+                                  .Arg<ffi::AnyBuffer>()  // seqlens
+                                  .Arg<ffi::AnyBuffer>()  // o
+                                  .Arg<ffi::AnyBuffer>()  // lse
+                                  .Arg<ffi::AnyBuffer>()  // dout
+                                  .Ret<ffi::AnyBuffer>()  // dq
+                                  .Ret<ffi::AnyBuffer>()  // dk
+                                  .Ret<ffi::AnyBuffer>()  // dv
+                                  .Ret<ffi::AnyBuffer>()  // scratch
+                                  .Attr<float>("scale")
+                                  .Attr<float>("dropout_p")
+                                  .Attr<bool>("causal")
+                                  .Attr<int64_t>("seed")
+                                  .Attr<bool>("bias_group"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(fa2_dropout_mask_ffi, DropoutMaskImpl,
+                              ffi::Ffi::Bind()
+                                  .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Ret<ffi::AnyBuffer>()  // keep
+                                  .Attr<float>("dropout_p")
+                                  .Attr<int64_t>("seed"));

@@ -22,6 +22,7 @@ import typing as tp
 import torch
 
 from . import _lib
+from ._checks import check_shapes  # noqa: F401  (re-exported)
 from ._lib import FA2_BF16, FA2_FP16, FA2_FP32, Fa2Tensor
 
 _DTYPES = {torch.float16: FA2_FP16, torch.bfloat16: FA2_BF16}
@@ -45,45 +46,6 @@ def _usable(x: torch.Tensor) -> torch.Tensor:
 	if x.stride(3) != 1 or any(s % 8 for s in x.stride()[:3]) or x.data_ptr() % 16:
 		return x.contiguous()
 	return x
-
-
-def check_shapes(q, k, v, bias, attention_mask):
-	"""Validation of `_fwd_attention_kernel_call` (_forward_triton.py:474-495) and
-	`calc_bias_strides` (_utils.py:151-193), with the reference's messages."""
-	batch, QSeq, nheads_q, head_dim = q.shape
-	_, KSeq, nheads_kv, _ = k.shape
-	expected_kv_shape = (batch, KSeq, nheads_kv, head_dim)
-	if attention_mask is not None:
-		assert bias is None, "Attention mask is not supported along with attention bias. Just use bias instead."
-		assert QSeq == KSeq, "Attention mask is not supported with QSeq != KSeq"
-	assert tuple(k.shape) == expected_kv_shape, (
-		f"key shape is k.shape = {tuple(k.shape)} and we excepted it to be like expected_kv_shape = {expected_kv_shape}"
-	)
-	assert tuple(v.shape) == expected_kv_shape, (
-		f"value shape is v.shape = {tuple(v.shape)} and we excepted it to be like expected_kv_shape = {expected_kv_shape}"
-	)
-	assert nheads_q % nheads_kv == 0, f"nheads_q = {nheads_q} is not divisible by nheads_kv ={nheads_kv}"
-	assert q.dtype == k.dtype == v.dtype, "All tensors must have the same type"
-	assert q.dtype in _DTYPES, "Only support fp16 and bf16"
-	if bias is not None:
-		if bias.shape[2] != QSeq or bias.shape[3] != KSeq:
-			raise ValueError(
-				f"Bias tensor has incompatible sequence dimensions. "
-				f"Expected shape [..., {QSeq}, {KSeq}], but got [..., {bias.shape[2]}, {bias.shape[3]}]. "
-				f"Full bias shape: {tuple(bias.shape)}"
-			)
-		if bias.shape[0] not in (1, batch):
-			raise ValueError(
-				f"Batch dimension mismatch in bias tensor. "
-				f"Expected either 1 (for broadcasting) or {batch} (batch size), "
-				f"but got {bias.shape[0]}. Consider reshaping your bias tensor."
-			)
-		if bias.shape[1] not in (1, nheads_q) and not (bias.shape[1] == nheads_kv):
-			raise ValueError(
-				f"Head dimension mismatch in bias tensor. "
-				f"Expected either 1 (for broadcasting) or {nheads_q} (number of heads), "
-				f"but got {bias.shape[1]}. Check that your bias tensor matches the model configuration."
-			)
 
 
 def _fill_common(p, q, k, v, bias, seqlens, scale, p_drop, causal, seed):

@@ -13,7 +13,7 @@ import threading
 FA2_FP16, FA2_BF16, FA2_FP32 = 1, 2, 3
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.environ.get("FA2_LIB", os.path.join(os.path.dirname(_HERE), "libfa2_hip.so"))
+LIB_PATH = os.path.join(os.path.dirname(_HERE), "libfa2_hip.so")
 
 
 class Fa2Tensor(ctypes.Structure):
