@@ -433,8 +433,8 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 // ---------------------------------------------------------------------------
 // dQ
 // ---------------------------------------------------------------------------
-template <typename T, int D, int NW, int QB, bool BIAS, bool DROP>
-__global__ __launch_bounds__(NW * 64) void bwd_dq_kernel(const KArgs a) {
+template <typename T, int D, int NW, int QB, int WPS, bool BIAS, bool DROP>
+__global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 	typedef typename T::V8 V8;
 	constexpr int BM = NW * QB * 32;
 	constexpr int BN = kFwdBN;
@@ -583,18 +583,28 @@ __global__ __launch_bounds__(NW * 64) void bwd_dq_kernel(const KArgs a) {
 			for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
 				for (int i = 0; i < 16; ++i) s[qb][i] = dp[qb][i] = 0.f;
+			__builtin_amdgcn_sched_barrier(0);
 #pragma unroll
 			for (int ks = 0; ks < KS; ++ks) {
 				V8 ka = *(const FA2_LDS V8*)(kt + koff[ks] + kb * (32 * D * 2));
 #pragma unroll
 				for (int qb = 0; qb < QB; ++qb) s[qb] = mfma32(ka, qf[qb][ks], s[qb]);
-			}
-#pragma unroll
-			for (int ks = 0; ks < KS; ++ks) {
 				V8 va = *(const FA2_LDS V8*)(vt + koff[ks] + kb * (32 * D * 2));
 #pragma unroll
 				for (int qb = 0; qb < QB; ++qb) dp[qb] = mfma32(va, dof[qb][ks], dp[qb]);
 			}
+			// issue order: a few fragment reads ahead, then one read per product
+			{
+				constexpr int NR = 2 * KS, PF = NR < 8 ? NR : 8;
+				__builtin_amdgcn_sched_group_barrier(0x100, PF, 0);
+#pragma unroll
+				for (int i = 0; i < NR - PF; ++i) {
+					__builtin_amdgcn_sched_group_barrier(0x008, QB, 0);
+					__builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+				}
+				__builtin_amdgcn_sched_group_barrier(0x008, PF * QB, 0);
+			}
+			__builtin_amdgcn_sched_barrier(0);
 			// K^T fragments for dQ^T += K^T dS^T, issued ahead of the elementwise math
 			constexpr bool BOTH_EARLY = DB <= 4;
 			u32x4 kfr[2][DB];
@@ -711,6 +721,7 @@ struct BwdCfg {
 	// dQ: 4 waves x QB x 32 rows
 	static constexpr int DQ_NW = D <= 128 ? 8 : 4;
 	static constexpr int DQ_QB = 1;
+	static constexpr int DQ_WPS = 1;
 	static constexpr int DQ_BM = DQ_NW * DQ_QB * 32;
 };
 
@@ -732,7 +743,7 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 	if (a.stages & 4) {
 		a.mtiles = (a.Sq + C::DQ_BM - 1) / C::DQ_BM;
 		dim3 grid((unsigned)(a.mtiles * a.B * a.Hq)), block(C::DQ_NW * 64);
-		hipLaunchKernelGGL((bwd_dq_kernel<T, D, C::DQ_NW, C::DQ_QB, BIAS, DROP>), grid, block, 0, s, a);
+		hipLaunchKernelGGL((bwd_dq_kernel<T, D, C::DQ_NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP>), grid, block, 0, s, a);
 	}
 	return hipGetLastError();
 }

@@ -80,8 +80,8 @@ FA2_DEV f32x4 load_bias4(const char* rowp, int col, int dtype, bool vec_ok, int 
 	return out;
 }
 
-template <typename T, int D, int NW, int QB, bool BIAS, bool DROP>
-__global__ __launch_bounds__(NW * 64) void fwd_kernel(const KArgs a) {
+template <typename T, int D, int NW, int QB, int WPS, bool BIAS, bool DROP>
+__global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 	typedef typename T::V8 V8;
 	constexpr int BM = NW * QB * 32;
 	constexpr int BN = kFwdBN;
@@ -240,6 +240,7 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const KArgs a) {
 			for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
 				for (int i = 0; i < 16; ++i) s[kb][qb][i] = 0.f;
+		__builtin_amdgcn_sched_barrier(0);
 #pragma unroll
 		for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
@@ -248,6 +249,19 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const KArgs a) {
 #pragma unroll
 				for (int qb = 0; qb < QB; ++qb) s[kb][qb] = mfma32(kf, qf[qb][ks], s[kb][qb]);
 			}
+		// issue order: a few fragment reads ahead, then one read per product, so that the
+		// LDS latency is paid once per tile instead of once per product
+		{
+			constexpr int NR = KS * KB, PF = NR < 8 ? NR : 8;
+			__builtin_amdgcn_sched_group_barrier(0x100, PF, 0);
+#pragma unroll
+			for (int i = 0; i < NR - PF; ++i) {
+				__builtin_amdgcn_sched_group_barrier(0x008, QB, 0);
+				__builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+			}
+			__builtin_amdgcn_sched_group_barrier(0x008, PF * QB, 0);
+		}
+		__builtin_amdgcn_sched_barrier(0);
 
 		// V fragments for O^T += V^T P^T, fetched in batches of NF; the first batch is in
 		// flight during the softmax, each further one during the products of the previous.
@@ -421,8 +435,11 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const KArgs a) {
 
 template <typename T, int D>
 struct FwdCfg {
+	// D <= 128: 8 waves, two per SIMD (<= 256 registers each): while one waits on LDS or
+	// on a matrix product the other issues.  D = 256 needs the whole register file.
 	static constexpr int NW = D <= 128 ? 8 : 4;
 	static constexpr int QB = 1;
+	static constexpr int WPS = 1;
 	static constexpr int BM = NW * QB * 32;
 };
 
@@ -434,13 +451,13 @@ hipError_t launch_fwd_t(bool bias, bool drop, KArgs& a, hipStream_t s) {
 	a.xcd_remap = (groups % 8 == 0) ? 1 : 0;
 	dim3 grid((unsigned)(a.mtiles * a.B * a.Hq)), block(C::NW * 64);
 	if (bias && drop)
-		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, true, true>), grid, block, 0, s, a);
+		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, C::WPS, true, true>), grid, block, 0, s, a);
 	else if (bias)
-		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, true, false>), grid, block, 0, s, a);
+		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, C::WPS, true, false>), grid, block, 0, s, a);
 	else if (drop)
-		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, false, true>), grid, block, 0, s, a);
+		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, C::WPS, false, true>), grid, block, 0, s, a);
 	else
-		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, false, false>), grid, block, 0, s, a);
+		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, C::WPS, false, false>), grid, block, 0, s, a);
 	return hipGetLastError();
 }
 
