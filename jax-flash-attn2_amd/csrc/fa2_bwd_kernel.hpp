@@ -66,6 +66,10 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	constexpr int NT = NW * 64;
 	constexpr int TILE_BYTES = BMQ * D * 2;
 	constexpr int STAT_BYTES = BMQ * 4;
+	// Register files pinned by hand (K / V fragments and the dK / dV accumulators in AGPRs, the
+	// S / dP accumulators in VGPRs) when the AGPR file holds the former; the bias and dropout
+	// variants need the registers for other things and leave the choice to the compiler.
+	constexpr bool KV_AGPR = 2 * KS * 4 + 2 * DB * 16 <= 256 && !BIAS && !DROP;
 
 	// Q[0] Q[1] dO[0] dO[1] | lse[0] lse[1] delta[0] delta[1]
 	__shared__ __attribute__((aligned(1024))) char smem[4 * TILE_BYTES + 4 * STAT_BYTES];
@@ -139,14 +143,18 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 
 	const float c1 = BIAS ? a.scale : a.scale * kLog2e;
 
-	auto issue_tile = [&](int step, FA2_LDS char* qdst, FA2_LDS char* dodst) {
+	TileLoader<D, BMQ, NT> qload, doload;
+	qload.init(a.q.ss, tid);
+	doload.init(a.dout.ss, tid);
+	// start the copies of streamed tile `step` (rows beyond Sq are fetched from the last valid row)
+	auto issue_tile = [&](int step, FA2_LDS char* qdst, FA2_LDS char* dodst) __attribute__((always_inline)) {
 		int hq = hk * r + step / nq;
 		int m0 = (q_lo + step % nq) * BMQ;
 		int rows = a.Sq - m0 < BMQ ? a.Sq - m0 : BMQ;
 		const char* qb_ = a.q.ptr + (int64_t)b * a.q.sb + (int64_t)hq * a.q.sh + (int64_t)m0 * a.q.ss;
 		const char* db_ = a.dout.ptr + (int64_t)b * a.dout.sb + (int64_t)hq * a.dout.sh + (int64_t)m0 * a.dout.ss;
-		tile_load_async<D, BMQ, NT>(qdst, qb_, a.q.ss, rows, tid);
-		tile_load_async<D, BMQ, NT>(dodst, db_, a.dout.ss, rows, tid);
+		qload.load(qdst, qb_, a.q.ss, rows, tid);
+		doload.load(dodst, db_, a.dout.ss, rows, tid);
 	};
 	// per-row statistics of a tile: thread t < BMQ fetches lse, t in [BMQ, 2 BMQ) fetches delta
 	auto fetch_stat = [&](int step) -> float {
@@ -192,7 +200,8 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 
 	// One streamed tile of BMQ query rows of q-head hq.  MASKED = some (row, key)
 	// of this wave's 32 keys x BMQ rows is masked.
-	auto tile_body = [&](auto masked_tag, const FA2_LDS char* qt, const FA2_LDS char* dot, int buf, int hq, int m0) {
+	auto tile_body = [&](auto masked_tag, const FA2_LDS char* qt, const FA2_LDS char* dot, int buf, int hq, int m0)
+	                     __attribute__((always_inline)) {
 		constexpr bool MASKED = decltype(masked_tag)::value;
 		const FA2_LDS char* lse_s = stat + buf * STAT_BYTES;
 		const FA2_LDS char* del_s = stat + (2 + buf) * STAT_BYTES;
@@ -208,139 +217,257 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		//   B(i): P_i, dS_i from S_i, dP_i, lse, delta      (elementwise, 16 values per lane)
 		//   C(i): dV^T += dO_i^T P_i, dK^T += Q_i^T dS_i   (4 DB matrix products)
 		// software-pipelined: pipeline stage k runs A(k), B(k-1) and C(k-2) together, cut
-		// into NCH chunks.  Chunk c issues its share of the products of A(k) and C(k-2),
-		// then the transposed LDS reads that feed later products, then the elementwise
-		// math of EPC of the 16 values of B(k-1) - so the vector ALU works in the shadow
-		// of the matrix pipe.  A scheduling barrier after every chunk pins that order.
-		constexpr int NFR = 2 * DB;  // transposed fragments of one 16-row half of a block: (dO^T, Q^T) x DB
-		constexpr int NCH = 8;            // chunks per stage
-		constexpr int EPC = 16 / NCH;     // elementwise values per chunk
+		// into NSLOT slots.  A slot issues one product of A(k), one of C(k-2), the LDS reads
+		// of the fragments that the slot PA places further on will use (so every read has PA
+		// slots to complete and the LDS traffic is spread evenly), and its share of the
+		// elementwise math of B(k-1) - the vector ALU and the LDS work in the shadow of the
+		// matrix pipe.  A scheduling barrier after every slot pins that order.
+		constexpr int NSLOT = 2 * KS;     // = 4 DB
+		constexpr int PA = 4;             // read-ahead distance in slots
+		constexpr int RING = PA + 1;
+		static_assert(NSLOT % 16 == 0 || 16 % NSLOT == 0, "");
 		f32x16 s[2], dp[2];
-		V8 pb[2][2], sb[2][2];
-		u32x4 tfr[2][NFR];  // [half]
-		V8 qa[KS], da[KS];
+		u32x4 pbits[2][2], sbits[2][2];   // [block parity][16-row half]: P and dS packed to 16 bits
+		V8 afr[RING];                     // fragments of Q_i / dO_i for the products of A
+		u32x4 cfr[RING];                  // transposed fragments of dO_i / Q_i for the products of C
 		f32x4 lse4[4], del4[4];
-		f32x16 pd;  // P after dropout of the block in B (feeds dV); its S becomes dS (feeds dK)
 		float bv[BIAS ? 16 : 1];
 
-		auto load_A = [&](int qb) {
-#pragma unroll
-			for (int ks = 0; ks < KS; ++ks) {
-				qa[ks] = *(const FA2_LDS V8*)(qt + poff[ks] + qb * (32 * D * 2));
-				da[ks] = *(const FA2_LDS V8*)(dot + poff[ks] + qb * (32 * D * 2));
-			}
+		// fragment of product j of A(qb): even j -> Q (S), odd j -> dO (dP), k-step j / 2
+		auto issue_A = [&](int qb, int j) __attribute__((always_inline)) {
+			const FA2_LDS char* base = ((j & 1) ? dot : qt) + poff[j >> 1] + qb * (32 * D * 2);
+			afr[(qb * NSLOT + j) % RING] = *(const FA2_LDS V8*)base;
 		};
-		auto load_stats = [&](int qb) {
-#pragma unroll
-			for (int aa = 0; aa < 4; ++aa) {
-				lse4[aa] = *(const FA2_LDS f32x4*)(lse_s + (32 * qb + 8 * aa + 4 * g) * 4);
-				del4[aa] = *(const FA2_LDS f32x4*)(del_s + (32 * qb + 8 * aa + 4 * g) * 4);
-			}
-			if constexpr (BIAS) {
-#pragma unroll
-				for (int i = 0; i < 16; ++i) {
-					int row = m0 + 32 * qb + 8 * (i >> 2) + 4 * g + (i & 3);
-					row = row < a.Sq ? row : a.Sq - 1;
-					const char* pp = bias_base + (int64_t)row * a.bias_sm;
-					bv[i] = a.bias_dtype == 3 ? *(const float*)pp
-					        : a.bias_dtype == 2 ? (float)*(const __bf16*)pp
-					                            : (float)*(const _Float16*)pp;
-				}
-			}
-		};
-		// product j of A: even j -> S, odd j -> dP, k-step j / 2
-		auto mfma_A = [&](int j, f32x16& sa, f32x16& dpa) {
-			int ks = j >> 1;
-			if (j & 1)
-				dpa = mfma32(da[ks], vf[ks], dpa);
-			else
-				sa = mfma32(qa[ks], kf[ks], sa);
-		};
-		// product j of C: half j / (2 DB); inside a half even -> dV, odd -> dK, d-block (j % (2 DB)) / 2
-		auto mfma_C = [&](int j, V8(&pbi)[2], V8(&sbi)[2]) {
+		// fragment of product j of C(qb): half j / (2 DB); inside a half even -> dO^T (dV), odd -> Q^T (dK)
+		auto issue_C = [&](int qb, int j) __attribute__((always_inline)) {
 			int hf = j / (2 * DB), rr = j % (2 * DB), db = rr >> 1;
-			if (rr & 1)
-				dk[db] = mfma32(as_frag<T>(tfr[hf][DB + db]), sbi[hf], dk[db]);
-			else
-				dv[db] = mfma32(as_frag<T>(tfr[hf][db]), pbi[hf], dv[db]);
+			const FA2_LDS char* base = ((rr & 1) ? qt : dot) + qb * (32 * D * 2);
+			cfr[(qb * NSLOT + j) % RING] = lds_tr_issue_rt<D>(base + toff[db][0], base + toff[db][1], hf);
 		};
-		// transposed fragment j of half hf of block qb: j < DB -> dO^T block j, else Q^T block j - DB
-		auto issue_tr = [&](int qb, int hf, int j, u32x4(&dst)[NFR]) {
-			const FA2_LDS char* base = (j < DB ? dot : qt) + qb * (32 * D * 2);
-			int db = j < DB ? j : j - DB;
-			dst[j] = lds_tr_issue_rt<D>(base + toff[db][0], base + toff[db][1], hf);
+		// statistics of rows 8 aa + 4 g .. + 3 of block qb
+		auto issue_stat = [&](int qb, int aa) __attribute__((always_inline)) {
+			lse4[aa] = *(const FA2_LDS f32x4*)(lse_s + (32 * qb + 8 * aa + 4 * g) * 4);
+			del4[aa] = *(const FA2_LDS f32x4*)(del_s + (32 * qb + 8 * aa + 4 * g) * 4);
 		};
-		// value i of B(qb)
-		auto elem_B = [&](int qb, int i, f32x16& sa, f32x16& dpa) {
-			int row = m0 + 32 * qb + 8 * (i >> 2) + 4 * g + (i & 3);
-			float lse = lse4[i >> 2][i & 3], del = del4[i >> 2][i & 3];
-			float p;
-			if constexpr (BIAS)
-				p = exp2_fast((__builtin_fmaf(sa[i], c1, bv[i]) - lse) * kLog2e);
-			else
-				p = exp2_fast(__builtin_fmaf(sa[i], c1, -lse));
-			if constexpr (MASKED) {
-				bool ok = row < sq_eff && jcol < sk_eff && (!a.causal || jcol <= row + off);
-				p = ok ? p : 0.f;
+		// statistics of the quads whose phase 0 runs in slot j
+		auto issue_stat_for_slot = [&](int qb, int j) __attribute__((always_inline)) {
+			if constexpr (NSLOT >= 16) {
+				if (j % (NSLOT / 4) == 0) issue_stat(qb, j / (NSLOT / 4));
+			} else {
+				constexpr int QPS = 16 / NSLOT;
+				if (j % 4 == 0)
+					for (int e = 0; e < QPS; ++e) issue_stat(qb, (j / 4) * QPS + e);
 			}
-			float pdrop = p, dpe = dpa[i];
+		};
+		auto load_bias = [&](int qb, int i) __attribute__((always_inline)) {
+			if constexpr (BIAS) {
+				int row = m0 + 32 * qb + 8 * (i >> 2) + 4 * g + (i & 3);
+				row = row < a.Sq ? row : a.Sq - 1;
+				const char* pp = bias_base + (int64_t)row * a.bias_sm;
+				bv[i] = a.bias_dtype == 3 ? *(const float*)pp
+				        : a.bias_dtype == 2 ? (float)*(const __bf16*)pp
+				                            : (float)*(const _Float16*)pp;
+			}
+		};
+		auto mfma_A = [&](int qb, int j, f32x16& sa, f32x16& dpa) __attribute__((always_inline)) {
+			int ks = j >> 1, r = (qb * NSLOT + j) % RING;
+			if constexpr (KV_AGPR) {
+				if (j == 0)
+					mfma32_vz<true>(sa, afr[r], kf[ks]);
+				else if (j == 1)
+					mfma32_vz<true>(dpa, afr[r], vf[ks]);
+				else if (j & 1)
+					mfma32_va<true>(dpa, afr[r], vf[ks]);
+				else
+					mfma32_va<true>(sa, afr[r], kf[ks]);
+			} else {
+				// too many registers to pin: leave the register files to the compiler
+				f32x16 zero;
+#pragma unroll
+				for (int i = 0; i < 16; ++i) zero[i] = 0.f;
+				if (j & 1)
+					dpa = mfma32(afr[r], vf[ks], j == 1 ? zero : dpa);
+				else
+					sa = mfma32(afr[r], kf[ks], j == 0 ? zero : sa);
+			}
+		};
+		auto mfma_C = [&](int qb, int j, u32x4(&pbi)[2], u32x4(&sbi)[2]) __attribute__((always_inline)) {
+			int hf = j / (2 * DB), rr = j % (2 * DB), db = rr >> 1, r = (qb * NSLOT + j) % RING;
+			if constexpr (KV_AGPR) {
+				if (rr & 1)
+					mfma32_aa(dk[db], as_frag<T>(cfr[r]), as_frag<T>(sbi[hf]));
+				else
+					mfma32_aa(dv[db], as_frag<T>(cfr[r]), as_frag<T>(pbi[hf]));
+			} else {
+				if (rr & 1)
+					dk[db] = mfma32(as_frag<T>(cfr[r]), as_frag<T>(sbi[hf]), dk[db]);
+				else
+					dv[db] = mfma32(as_frag<T>(cfr[r]), as_frag<T>(pbi[hf]), dv[db]);
+			}
+		};
+		// B(qb) as 16 micro-steps: quad q (values 4q .. 4q+3, rows 8q + 4g + e) goes through
+		//   phase 0: x = S c1 - lse, y = dP - delta     phase 1: P = exp2(x) (mask, dropout)
+		//   phase 2: dS = P y                            phase 3: pack P and dS to 16 bits
+		// Every micro-step is four independent operations per instruction kind, and the phases
+		// of a quad sit in different slots: a vector-ALU result is only consumed many cycles
+		// after it was issued (back-to-back dependent vector operations would each wait for
+		// the previous one's full pipeline latency).
+		float bx[4][4], by[4][4];
+		// dropout keep bits of a quad (bit e = value 4q + e), produced one value per slot while
+		// the previous quad is processed: one Philox call at a time keeps its registers few
+		uint32_t keepw[4] = {0u, 0u, 0u, 0u};
+		auto keep_bit = [&](int qb, int q, int e) __attribute__((always_inline)) {
 			if constexpr (DROP) {
+				int row = m0 + 32 * qb + 8 * q + 4 * g + e;
 				u32x4 rnd = philox4x32_10((uint32_t)(jcol >> 2), (uint32_t)row, (uint32_t)hq, (uint32_t)b, a.drop_k0, a.drop_k1);
 				uint32_t word = rnd[0];
 				word = (jcol & 3) == 1 ? rnd[1] : word;
 				word = (jcol & 3) == 2 ? rnd[2] : word;
 				word = (jcol & 3) == 3 ? rnd[3] : word;
-				bool keep = word >= a.drop_thr;
-				pdrop = keep ? p : 0.f;
-				dpe = keep ? dpe * a.drop_inv_keep : 0.f;
+				uint32_t bit = word >= a.drop_thr ? (1u << e) : 0u;
+				keepw[q & 3] = e == 0 ? bit : (keepw[q & 3] | bit);
 			}
-			pd[i] = pdrop;
-			sa[i] = p * (dpe - del);
 		};
-		auto pack_B = [&](int hf, f32x16& sa, V8(&pbo)[2], V8(&sbo)[2]) {
-			pbo[hf] = pack8<T>(pd[8 * hf + 0], pd[8 * hf + 1], pd[8 * hf + 2], pd[8 * hf + 3], pd[8 * hf + 4], pd[8 * hf + 5],
-			                   pd[8 * hf + 6], pd[8 * hf + 7]);
-			sbo[hf] = pack8<T>(sa[8 * hf + 0], sa[8 * hf + 1], sa[8 * hf + 2], sa[8 * hf + 3], sa[8 * hf + 4], sa[8 * hf + 5],
-			                   sa[8 * hf + 6], sa[8 * hf + 7]);
+		auto micro_B = [&](int qb, int q, int phase, int e0, int e1, const f32x16& sa, const f32x16& dpa, u32x4(&pbo)[2], u32x4(&sbo)[2])
+		                   __attribute__((always_inline)) {
+			if (phase == 0) {
+#pragma unroll
+				for (int e = e0; e < e1; ++e) {
+					int i = 4 * q + e;
+					if constexpr (BIAS)
+						bx[q][e] = (__builtin_fmaf(sa[i], c1, bv[i]) - lse4[q][e]) * kLog2e;
+					else
+						bx[q][e] = __builtin_fmaf(sa[i], c1, -lse4[q][e]);
+				}
+			} else if (phase == 1) {
+#pragma unroll
+				for (int e = e0; e < e1; ++e) {
+					// dP is read here, not in phase 0: the last product of its chain is then at
+					// least two matrix products back
+					if constexpr (!DROP) by[q][e] = dpa[4 * q + e] - del4[q][e];
+					float p = exp2_fast(bx[q][e]);
+					int row = m0 + 32 * qb + 8 * q + 4 * g + e;
+					if constexpr (MASKED) {
+						bool ok = row < sq_eff && jcol < sk_eff && (!a.causal || jcol <= row + off);
+						p = ok ? p : 0.f;
+					}
+					bx[q][e] = p;
+					if constexpr (DROP) {
+						bool keep = (keepw[q & 3] >> e) & 1u;
+						// by = dP keep / (1 - p_drop) - delta ; bx keeps P, the dropped P goes to dV
+						by[q][e] = keep ? __builtin_fmaf(dpa[4 * q + e], a.drop_inv_keep, -del4[q][e]) : -del4[q][e];
+						bx[q][e] = keep ? p : -p;  // sign bit marks a dropped value (P >= 0)
+					}
+				}
+			} else if (phase == 2) {
+#pragma unroll
+				for (int e = e0; e < e1; ++e) by[q][e] = __builtin_fabsf(bx[q][e]) * by[q][e];
+			} else {
+				int hf = q >> 1, m = (q & 1) * 2;
+#pragma unroll
+				for (int e = e0; e < e1; e += 2) {
+					float p0 = bx[q][e], p1 = bx[q][e + 1];
+					if constexpr (DROP) {
+						p0 = p0 < 0.f ? 0.f : p0;
+						p1 = p1 < 0.f ? 0.f : p1;
+					}
+					pbo[hf][m + e / 2] = pack2<typename T::V2>(p0, p1);
+					sbo[hf][m + e / 2] = pack2<typename T::V2>(by[q][e], by[q][e + 1]);
+				}
+			}
 		};
 
-		auto stage = [&](auto k_tag) {
+		// reads that the first PA slots of stage 0 use
+#pragma unroll
+		for (int j = 0; j < PA; ++j) issue_A(0, j);
+
+		auto stage = [&](auto k_tag) __attribute__((always_inline)) {
 			constexpr int k = decltype(k_tag)::value;
-			constexpr bool HAS_C = k >= 2, HAS_A = k < QB, HAS_B = k >= 1 && k - 1 < QB;
-			__builtin_amdgcn_sched_barrier(0);
-			if constexpr (HAS_B) load_stats(k - 1);
-			if constexpr (HAS_A) {
-				load_A(k);
-#pragma unroll
-				for (int i = 0; i < 16; ++i) s[k & 1][i] = dp[k & 1][i] = 0.f;
-			}
+			constexpr bool HAS_A = k < QB, HAS_B = k >= 1 && k - 1 < QB, HAS_C = k >= 2 && k - 2 < QB;
+			constexpr bool NEXT_A = k + 1 < QB, NEXT_B = k + 1 >= 1 && k < QB, NEXT_C = k + 1 >= 2 && k - 1 < QB;
 			__builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-			for (int c = 0; c < NCH; ++c) {
-				if constexpr (HAS_A) {
-#pragma unroll
-					for (int j = c * (2 * KS) / NCH; j < (c + 1) * (2 * KS) / NCH; ++j) mfma_A(j, s[k & 1], dp[k & 1]);
-				}
-				if constexpr (HAS_C) {
-#pragma unroll
-					for (int j = c * (4 * DB) / NCH; j < (c + 1) * (4 * DB) / NCH; ++j) mfma_C(j, pb[k & 1], sb[k & 1]);
-					// second half of C(k-2)'s fragments: read during the first eight chunks, used in the last eight
-					if (c < NCH / 2) {
-#pragma unroll
-						for (int j = c * NFR / (NCH / 2); j < (c + 1) * NFR / (NCH / 2); ++j) issue_tr(k - 2, 1, j, tfr[1]);
+			for (int j = 0; j < NSLOT; ++j) {
+				// LDS reads for the slot PA places ahead (in this stage or the next one)
+				{
+					int jn = j + PA;
+					if (jn < NSLOT) {
+						if constexpr (HAS_A) issue_A(k, jn);
+						if constexpr (HAS_C) issue_C(k - 2, jn);
+						if constexpr (HAS_B) {
+							issue_stat_for_slot(k - 1, jn);
+						}
+					} else {
+						int jj = jn - NSLOT;
+						if constexpr (NEXT_A) issue_A(k + 1, jj);
+						if constexpr (NEXT_C) issue_C(k - 1, jj);
+						if constexpr (NEXT_B) {
+							issue_stat_for_slot(k, jj);
+						}
 					}
 				}
-				if constexpr (HAS_B) {
-					// first half of C(k-1)'s fragments, into the buffer C(k-2) has finished with
-					if (c >= NCH / 2) {
+				// first half of the slot: product of A, first half of the micro-step(s) of B;
+				// second half: product of C, second half of the micro-step(s) - each matrix
+				// product is followed by vector-ALU work, never directly by another product
+				auto b_half = [&](int e0, int e1) __attribute__((always_inline)) {
+					if constexpr (HAS_B) {
+						if constexpr (NSLOT >= 16) {
+							if (j % (NSLOT / 16) == NSLOT / 16 - 1) {
+								int ms = j / (NSLOT / 16);
+								if constexpr (BIAS) {
+									if (ms % 4 == 0)
+										for (int e = e0; e < e1; ++e) load_bias(k - 1, ms + e);
+								}
+								micro_B(k - 1, ms / 4, ms % 4, e0, e1, s[(k - 1) & 1], dp[(k - 1) & 1], pbits[(k - 1) & 1], sbits[(k - 1) & 1]);
+							}
+						} else {
+							// several quads share a slot, all in the same phase
+							constexpr int QPS = 16 / NSLOT;  // quads per slot
+							int grp = j / 4, phase = j % 4;
 #pragma unroll
-						for (int j = (c - NCH / 2) * NFR / (NCH / 2); j < (c - NCH / 2 + 1) * NFR / (NCH / 2); ++j)
-							issue_tr(k - 1, 0, j, tfr[0]);
+							for (int e = 0; e < QPS; ++e) {
+								int q = grp * QPS + e;
+								if constexpr (BIAS) {
+									if (phase == 0)
+										for (int z = e0; z < e1; ++z) load_bias(k - 1, 4 * q + z);
+								}
+								micro_B(k - 1, q, phase, e0, e1, s[(k - 1) & 1], dp[(k - 1) & 1], pbits[(k - 1) & 1], sbits[(k - 1) & 1]);
+							}
+						}
 					}
-#pragma unroll
-					for (int e = 0; e < EPC; ++e) elem_B(k - 1, c * EPC + e, s[(k - 1) & 1], dp[(k - 1) & 1]);
-					if (c == NCH / 2 - 1) pack_B(0, s[(k - 1) & 1], pb[(k - 1) & 1], sb[(k - 1) & 1]);
-					if (c == NCH - 1) pack_B(1, s[(k - 1) & 1], pb[(k - 1) & 1], sb[(k - 1) & 1]);
+				};
+				if constexpr (HAS_A) mfma_A(k, j, s[k & 1], dp[k & 1]);
+				// the vector-ALU work below must not move above the product: for the products
+				// issued as inline assembly that order is what keeps a read of S / dP at least
+				// two matrix products away from the last product of its chain
+				if constexpr (HAS_A && HAS_B) __builtin_amdgcn_sched_barrier(0);
+				b_half(0, 2);
+				if constexpr (HAS_A && HAS_C) __builtin_amdgcn_sched_barrier(0);
+				if constexpr (HAS_C) mfma_C(k - 2, j, pbits[k & 1], sbits[k & 1]);
+				b_half(2, 4);
+				if constexpr (HAS_B && DROP) {
+					if constexpr (NSLOT >= 16) {
+						if (j % (NSLOT / 16) == NSLOT / 16 - 1) {
+							int ms = j / (NSLOT / 16);
+							if (ms + 4 < 16) keep_bit(k - 1, (ms + 4) / 4, ms % 4);
+						}
+					} else {
+						constexpr int QPS = 16 / NSLOT;
+						for (int e = 0; e < QPS; ++e) {
+							int q = (j / 4) * QPS + e;
+							if (q + QPS < 4) keep_bit(k - 1, q + QPS, j % 4);
+						}
+					}
+				}
+				if constexpr (NEXT_B && DROP) {
+					// keep bits of the first quad(s) of the next block, in the last slots of this stage
+					if constexpr (NSLOT >= 16) {
+						if (j >= NSLOT - 4 * (NSLOT / 16) && (j - (NSLOT - 4 * (NSLOT / 16))) % (NSLOT / 16) == 0)
+							keep_bit(k, 0, (j - (NSLOT - 4 * (NSLOT / 16))) / (NSLOT / 16));
+					} else {
+						if (j >= NSLOT - 4)
+							for (int e = 0; e < 16 / NSLOT; ++e) keep_bit(k, e, j - (NSLOT - 4));
+					}
 				}
 				__builtin_amdgcn_sched_barrier(0);
 			}
@@ -373,8 +500,8 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 				    // statistics first: loads return in order, so waiting for this small load later
 				    // does not wait for the tile copies issued after it
 				    next_stat = fetch_stat(step + 1);
-				    issue_tile(step + 1, nq_, ndo);
 			    }
+			    if (has_next) issue_tile(step + 1, nq_, ndo);
 		    },
 		    [&](const FA2_LDS char* qt, const FA2_LDS char* dot) {
 			    const int hq = hk * r + step / nq;
@@ -409,6 +536,8 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		for (int i = i_full; i < nq; ++i) run_step(std::true_type{}, base + i);
 	}
 
+	// the last matrix products (issued as inline assembly) must have written dk / dv
+	asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 	// epilogue: lane owns key jcol, four consecutive d per store
 	if (jcol < a.Sk) {
 		char* dkp = a.dk.ptr + (int64_t)b * a.dk.sb + (int64_t)hk * a.dk.sh + (int64_t)jcol * a.dk.ss;
@@ -509,10 +638,13 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 
 	const char* kbase = a.k.ptr + (int64_t)b * a.k.sb + (int64_t)hk * a.k.sh;
 	const char* vbase = a.v.ptr + (int64_t)b * a.v.sb + (int64_t)hk * a.v.sh;
+	TileLoader<D, BN, NT> kload, vload;
+	kload.init(a.k.ss, tid);
+	vload.init(a.v.ss, tid);
 	if (ntiles > 0) {
 		int rows = sk_eff < BN ? sk_eff : BN;
-		tile_load_async<D, BN, NT>(lds, kbase, a.k.ss, rows, tid);
-		tile_load_async<D, BN, NT>(lds + 2 * TILE_BYTES, vbase, a.v.ss, rows, tid);
+		kload.load(lds, kbase, a.k.ss, rows, tid);
+		vload.load(lds + 2 * TILE_BYTES, vbase, a.v.ss, rows, tid);
 	}
 
 	V8 qf[QB][KS], dof[QB][KS];
@@ -673,8 +805,8 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 			    if (t + 1 < ntiles) {
 				    int n1 = n0 + BN;
 				    int rows = sk_eff - n1 < BN ? sk_eff - n1 : BN;
-				    tile_load_async<D, BN, NT>(nk, kbase + (int64_t)n1 * a.k.ss, a.k.ss, rows, tid);
-				    tile_load_async<D, BN, NT>(nv, vbase + (int64_t)n1 * a.v.ss, a.v.ss, rows, tid);
+				    kload.load(nk, kbase + (int64_t)n1 * a.k.ss, a.k.ss, rows, tid);
+				    vload.load(nv, vbase + (int64_t)n1 * a.v.ss, a.v.ss, rows, tid);
 			    }
 		    },
 		    [&](const FA2_LDS char* kt, const FA2_LDS char* vt) {

@@ -51,6 +51,54 @@ FA2_DEV f32x16 mfma32(f16x8 a, f16x8 b, f32x16 c) {
 	return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
 }
 
+// The same product issued through inline assembly so that the register file of
+// every operand is fixed by the constraint: accumulators that only matrix
+// products touch (and operands that stay for the whole kernel) live in AGPRs,
+// accumulators that the vector ALU consumes live in VGPRs.  Left to itself the
+// register allocator puts those into AGPRs as well and copies each value out
+// with v_accvgpr_read before the vector ALU can use it.
+// The compiler does not know these statements are matrix products, so it adds
+// no wait states for them: the caller keeps a vector-ALU read of a result at
+// least two further matrix products away from the product that wrote it.
+//   mfma32_vz: C(VGPR) = A(VGPR) * B(AGPR)            first product of a chain
+//   mfma32_va: C(VGPR) += A(VGPR) * B(AGPR)
+//   mfma32_aa: C(AGPR) += A(VGPR) * B(VGPR)
+// BA: the B operand lives in an AGPR (else in a VGPR)
+template <bool BA>
+FA2_DEV void mfma32_vz(f32x16& c, bf16x8 a, bf16x8 b) {
+	if constexpr (BA)
+		asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
+	else
+		asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
+}
+template <bool BA>
+FA2_DEV void mfma32_vz(f32x16& c, f16x8 a, f16x8 b) {
+	if constexpr (BA)
+		asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
+	else
+		asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
+}
+template <bool BA>
+FA2_DEV void mfma32_va(f32x16& c, bf16x8 a, bf16x8 b) {
+	if constexpr (BA)
+		asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+	else
+		asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+}
+template <bool BA>
+FA2_DEV void mfma32_va(f32x16& c, f16x8 a, f16x8 b) {
+	if constexpr (BA)
+		asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+	else
+		asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+}
+FA2_DEV void mfma32_aa(f32x16& c, bf16x8 a, bf16x8 b) {
+	asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+FA2_DEV void mfma32_aa(f32x16& c, f16x8 a, f16x8 b) {
+	asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+
 template <typename V2>
 FA2_DEV uint32_t pack2(float a, float b) {
 	f32x2 f = {a, b};
@@ -183,6 +231,20 @@ FA2_DEV typename T::V8 as_frag(u32x4 x) {
 // swizzle is applied by choosing which global chunk each lane fetches.  Rows
 // at or beyond `rows_valid` are fetched from the last valid row instead (the
 // caller masks their scores), so no lane reads out of bounds.
+// One wave-level 64 x 16-byte direct global->LDS copy: lane i fetches 16 bytes at
+// `src` and they land at LDS byte address `wave_dst` + 16 i (`wave_dst` is
+// wave-uniform).  Issued through inline assembly on purpose: the compiler then
+// does not model the copy as an LDS access in flight.  If it did, every wait for
+// an LDS read (s_waitcnt lgkmcnt) issued while a copy is outstanding would
+// drain ALL outstanding LDS reads instead of only those older than the one
+// needed, which defeats reading fragments several products ahead.  Completion
+// is awaited explicitly with wait_async_loads() before the workgroup barrier
+// that publishes the tile.
+FA2_DEV void lds_dma16(const char* src, FA2_LDS char* wave_dst) {
+	uint32_t m = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)wave_dst);
+	asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(m) : "memory", "m0");
+}
+
 template <int D, int ROWS, int NTHREADS>
 FA2_DEV void tile_load_async(FA2_LDS char* tile, const char* gbase, int64_t stride_bytes, int rows_valid, int tid) {
 	constexpr int CPR = D / 8;  // 16-byte chunks per row
@@ -199,9 +261,66 @@ FA2_DEV void tile_load_async(FA2_LDS char* tile, const char* gbase, int64_t stri
 		int chunk = pchunk ^ swz<D>(row);
 		int grow = row < rows_valid ? row : rows_valid - 1;
 		const char* src = gbase + (int64_t)grow * stride_bytes + (chunk << 4);
-		__builtin_amdgcn_global_load_lds((const FA2_GLB void*)src, (FA2_LDS void*)(tile + slot0 * 16), 16, 0, 0);
+		lds_dma16(src, tile + slot0 * 16);
 	}
 }
+
+// The same copy with the addressing hoisted out of the loop that streams tiles:
+// init() computes, once, this lane's byte offsets inside a full tile; load() then
+// issues one instruction per 64 x 16 bytes from a wave-uniform tile base (SGPR
+// pair) plus that 32-bit lane offset.  Ragged tiles (fewer than ROWS valid rows)
+// and strides too large for 32-bit offsets take the general path above.
+FA2_DEV void lds_dma16_so(uint32_t lane_off, const char* uniform_base, FA2_LDS char* wave_dst) {
+	uint32_t m = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)wave_dst);
+	asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(uniform_base), "s"(m)
+	             : "m0");
+}
+
+template <int D, int ROWS, int NTHREADS>
+struct TileLoader {
+	static constexpr int CPR = D / 8;
+	static constexpr int TOTAL = ROWS * CPR;
+	static constexpr int NIT = TOTAL / NTHREADS;  // 64 x 16 byte pieces per wave and tile
+	static_assert(TOTAL % NTHREADS == 0, "tile must divide over the workgroup");
+	uint32_t off[NIT];
+	int rows_state;  // the offsets clamp rows to [0, rows_state)
+
+	// stride_bytes * ROWS must fit 31 bits (the launcher checks)
+	FA2_DEV void init(int64_t stride_bytes, int tid, int rows_valid = ROWS) {
+		rows_state = rows_valid;
+#pragma unroll
+		for (int it = 0; it < NIT; ++it) {
+			int slot = it * NTHREADS + tid;
+			int row = slot / CPR;
+			int chunk = (slot % CPR) ^ swz<D>(row);
+			int grow = row < rows_valid ? row : rows_valid - 1;
+			off[it] = (uint32_t)grow * (uint32_t)stride_bytes + (uint32_t)(chunk << 4);
+		}
+	}
+	// make the offsets fit a tile with rows_valid rows (wave-uniform; recomputes only on change)
+	FA2_DEV void fit(int64_t stride_bytes, int tid, int rows_valid) {
+		rows_valid = rows_valid < ROWS ? rows_valid : ROWS;
+		if (rows_valid != rows_state) init(stride_bytes, tid, rows_valid);
+	}
+	// a wave-uniform pointer as an explicitly scalar value
+	static FA2_DEV const char* uniform(const char* p) {
+		uint64_t gb = (uint64_t)p;
+		uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)gb), hi = __builtin_amdgcn_readfirstlane((uint32_t)(gb >> 32));
+		return (const char*)(((uint64_t)hi << 32) | lo);
+	}
+	// piece `it` (0 .. NIT-1) of the tile whose first row is at ub = uniform(address)
+	FA2_DEV void load_one(FA2_LDS char* tile, const char* ub, int it, int tid) const {
+		int wave_base = (tid >> 6) << 6;
+		lds_dma16_so(off[it], ub, tile + (it * NTHREADS + wave_base) * 16);
+	}
+	// whole tile; rows at or beyond rows_valid are fetched from the last valid row
+	FA2_DEV void load(FA2_LDS char* tile, const char* gbase, int64_t stride_bytes, int rows_valid, int tid) {
+		fit(stride_bytes, tid, rows_valid);
+		const char* ub = uniform(gbase);
+#pragma unroll
+		for (int it = 0; it < NIT; ++it) load_one(tile, ub, it, tid);
+	}
+};
 
 FA2_DEV void wait_async_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 

@@ -155,11 +155,14 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 	const char* kbase = a.k.ptr + (int64_t)b * a.k.sb + (int64_t)hk * a.k.sh;
 	const char* vbase = a.v.ptr + (int64_t)b * a.v.sb + (int64_t)hk * a.v.sh;
 
+	TileLoader<D, BN, NT> kload, vload;
+	kload.init(a.k.ss, tid);
+	vload.init(a.v.ss, tid);
 	// prologue: first K/V tile in flight while Q is fetched
 	if (ntiles > 0) {
 		int rows = sk_eff < BN ? sk_eff : BN;
-		tile_load_async<D, BN, NT>(lds, kbase, a.k.ss, rows, tid);
-		tile_load_async<D, BN, NT>(lds + 2 * TILE_BYTES, vbase, a.v.ss, rows, tid);
+		kload.load(lds, kbase, a.k.ss, rows, tid);
+		vload.load(lds + 2 * TILE_BYTES, vbase, a.v.ss, rows, tid);
 	}
 
 	// Q fragments (B operand of S^T): lane holds Q[row c][16ks + 8g .. +7]
@@ -383,8 +386,8 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 			    if (t + 1 < ntiles) {
 				    int n1 = n0 + BN;
 				    int rows = sk_eff - n1 < BN ? sk_eff - n1 : BN;
-				    tile_load_async<D, BN, NT>(nk, kbase + (int64_t)n1 * a.k.ss, a.k.ss, rows, tid);
-				    tile_load_async<D, BN, NT>(nv, vbase + (int64_t)n1 * a.v.ss, a.v.ss, rows, tid);
+				    kload.load(nk, kbase + (int64_t)n1 * a.k.ss, a.k.ss, rows, tid);
+				    vload.load(nv, vbase + (int64_t)n1 * a.v.ss, a.v.ss, rows, tid);
 			    }
 		    },
 		    [&](const FA2_LDS char* kt, const FA2_LDS char* vt) {
