@@ -88,6 +88,17 @@ def event_time_ms(fn, iters, torch):
 	return start.elapsed_time(stop) / iters
 
 
+def measured_traffic(workload, kernel):
+	"""HBM bytes per launch of `kernel` from the committed rocprofv3 FETCH_SIZE / WRITE_SIZE runs, or None."""
+	path = os.path.join(ROOT, "profiles", f"{workload}_traffic.json")
+	try:
+		with open(path) as f:
+			rec = json.load(f)
+	except (OSError, ValueError):
+		return None
+	return rec.get("hbm_bytes_per_launch") if rec.get("kernel") == kernel else None
+
+
 def cpu_baseline(w):
 	"""Reference JAX-platform algorithm (NumPy restatement) on a bounded sample of the workload."""
 	sys.path.insert(0, os.path.join(ROOT, "oracle"))
@@ -130,6 +141,9 @@ def main():
 	ap.add_argument("--warmup", type=int, default=3)
 	ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
 	ap.add_argument("--no-cpu-baseline", action="store_true")
+	ap.add_argument("--copy-calibration", action="store_true",
+	                help="also run a plain 1 GiB device copy (known traffic) so that rocprofv3 FETCH_SIZE / WRITE_SIZE "
+	                     "readings of the attention kernels can be scaled")
 	args = ap.parse_args()
 	if args.gpus != 1:
 		print("bench.py: this build measures ONE GPU; --gpus N with N > 1 is not supported "
@@ -153,6 +167,14 @@ def main():
 		plan.forward()
 		if w["bwd"]:
 			plan.backward()
+
+	if args.copy_calibration:
+		src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+		dst = torch.empty_like(src)
+		for _ in range(3):
+			dst.copy_(src)
+		torch.cuda.synchronize()
+		del src, dst
 
 	for _ in range(args.warmup):
 		step()
@@ -189,7 +211,7 @@ def main():
 		"peak": peak,
 		"unit": "TFLOP/s",
 		"frac": achieved / peak,
-		"traffic": None,
+		"traffic": measured_traffic(args.workload, dom),
 		"kernel_ms": {n: round(t, 4) for n, t in kern.items()},
 		"kernel_tflops": {n: round(alg[n] / (kern[n] * 1e-3) / 1e12, 1) for n in kern if n in alg},
 	}

@@ -40,7 +40,8 @@ enum {
 	FA2_EINVAL_SHAPE = -3,    /* non-positive dimension, or scale not finite and > 0 */
 	FA2_EINVAL_HEADS = -4,    /* Hq % Hkv != 0 (flash_attention.py:189-193)      */
 	FA2_EINVAL_PTR = -5,      /* required pointer is NULL or not 16-byte aligned */
-	FA2_EINVAL_STRIDE = -6,   /* stride not a multiple of 8 elements             */
+	FA2_EINVAL_STRIDE = -6,   /* stride not a multiple of 8 elements, or a sequence
+	                             stride that is negative or above 2^31 / 256 elements */
 	FA2_EINVAL_DROPOUT = -7,  /* p_drop outside [0, 1)                           */
 	FA2_EINVAL_BIAS = -8,     /* bias dtype / stride invalid                     */
 	FA2_EINVAL_MASK = -9,     /* seqlens given together with bias or with Sq != Sk

@@ -19,6 +19,8 @@ int check_tensor(const fa2_tensor& t, bool required) {
 	if (!aligned16(t.ptr)) return FA2_EINVAL_PTR;
 	// 16-byte vector access along D needs every row start 16-byte aligned
 	if (t.stride_b % 8 || t.stride_s % 8 || t.stride_h % 8) return FA2_EINVAL_STRIDE;
+	// the tile copies address the rows of a tile (up to 128) with 32-bit byte offsets
+	if (t.stride_s < 0 || t.stride_s > (int64_t)0x7fffffff / (2 * 128)) return FA2_EINVAL_STRIDE;
 	return FA2_OK;
 }
 
@@ -191,7 +193,7 @@ const char* fa2_strerror(int code) {
 		case FA2_EINVAL_SHAPE: return "dimensions must be positive and the softmax scale finite and positive";
 		case FA2_EINVAL_HEADS: return "query heads must be divisible by key/value heads";
 		case FA2_EINVAL_PTR: return "required pointer is NULL or misaligned";
-		case FA2_EINVAL_STRIDE: return "batch/sequence/head strides must be multiples of 8 elements";
+		case FA2_EINVAL_STRIDE: return "strides must be multiples of 8 elements and the sequence stride in [0, 2^31 / 256] elements";
 		case FA2_EINVAL_DROPOUT: return "dropout probability must be in [0, 1)";
 		case FA2_EINVAL_BIAS: return "bias dtype or strides invalid";
 		case FA2_EINVAL_MASK: return "Attention mask is not supported along with attention bias or with QSeq != KSeq";

@@ -291,7 +291,9 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 		V8 pf[QB][BN / 16];
 #pragma unroll
 		for (int qb = 0; qb < QB; ++qb) {
-			float mx = -INFINITY;
+			// four independent partial maxima (and, below, partial sums): a chain of dependent
+			// vector-ALU operations pays the full pipeline latency at every link
+			float mx4[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
 #pragma unroll
 			for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
@@ -303,8 +305,9 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 						x = j <= jmax[qb] ? x : -INFINITY;
 					}
 					s[kb][qb][i] = x;
-					mx = __builtin_fmaxf(mx, x);
+					mx4[i & 3] = __builtin_fmaxf(mx4[i & 3], x);
 				}
+			float mx = __builtin_fmaxf(__builtin_fmaxf(mx4[0], mx4[1]), __builtin_fmaxf(mx4[2], mx4[3]));
 			mx = pair_max(mx);
 			// to the softmax domain (log2 units without bias, natural units with bias)
 			if constexpr (!BIAS) mx = mx * c1;  // c1 > 0 is checked by the launcher
@@ -322,17 +325,17 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 			}
 			const float m_use = mrow[qb] == -INFINITY ? 0.f : mrow[qb];
 			const float nm = BIAS ? -m_use * kLog2e : -m_use;
-			float lsum = 0.f;
+			float ls4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
 			for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
 				for (int i = 0; i < 16; ++i) {
 					float p = BIAS ? exp2_fast(__builtin_fmaf(s[kb][qb][i] - m_use, kLog2e, 0.f))
 					               : exp2_fast(__builtin_fmaf(s[kb][qb][i], c1, nm));
-					lsum += p;
+					ls4[i & 3] += p;
 					s[kb][qb][i] = p;
 				}
-			lrow[qb] += lsum;
+			lrow[qb] += (ls4[0] + ls4[1]) + (ls4[2] + ls4[3]);
 			if constexpr (DROP) {
 #pragma unroll
 				for (int kb = 0; kb < KB; ++kb)

@@ -89,6 +89,8 @@ def test_validate_accepts_good_params():
 		(lambda p: setattr(p.q, "ptr", 0), -5),
 		(lambda p: setattr(p.k, "ptr", 0x10008), -5),
 		(lambda p: setattr(p.v, "stride_s", 1028), -6),
+		(lambda p: setattr(p.k, "stride_s", 1 << 24), -6),  # rows of a tile no longer within 32-bit byte offsets
+		(lambda p: setattr(p.q, "stride_s", -1024), -6),
 		(lambda p: setattr(p, "p_drop", 1.0), -7),
 		(lambda p: setattr(p, "p_drop", -0.1), -7),
 		(lambda p: (setattr(p, "bias", 0x40000), setattr(p, "bias_dtype", 7)), -8),
