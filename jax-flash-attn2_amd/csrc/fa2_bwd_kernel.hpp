@@ -56,7 +56,8 @@ __global__ __launch_bounds__(256) void bwd_delta_kernel(const KArgs a) {
 // ---------------------------------------------------------------------------
 // dK / dV
 // ---------------------------------------------------------------------------
-template <typename T, int D, int NW, int QB, bool BIAS, bool DROP>
+// BIAS_T: the bias has the element type of q / k / v (no run-time type dispatch per value)
+template <typename T, int D, int NW, int QB, bool BIAS, bool DROP, bool BIAS_T>
 __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	typedef typename T::V8 V8;
 	constexpr int BN = NW * 32;     // keys per workgroup
@@ -231,7 +232,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		V8 afr[RING];                     // fragments of Q_i / dO_i for the products of A
 		u32x4 cfr[RING];                  // transposed fragments of dO_i / Q_i for the products of C
 		f32x4 lse4[4], del4[4];
-		float bv[BIAS ? 16 : 1];
+		float bv[2][BIAS ? 16 : 1];       // [block parity]: bias values, fetched one stage ahead of their use
 
 		// fragment of product j of A(qb): even j -> Q (S), odd j -> dO (dP), k-step j / 2
 		auto issue_A = [&](int qb, int j) __attribute__((always_inline)) {
@@ -264,9 +265,23 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 				int row = m0 + 32 * qb + 8 * (i >> 2) + 4 * g + (i & 3);
 				row = row < a.Sq ? row : a.Sq - 1;
 				const char* pp = bias_base + (int64_t)row * a.bias_sm;
-				bv[i] = a.bias_dtype == 3 ? *(const float*)pp
-				        : a.bias_dtype == 2 ? (float)*(const __bf16*)pp
-				                            : (float)*(const _Float16*)pp;
+				if constexpr (BIAS_T)
+					bv[qb & 1][i] = (float)*(const typename T::E*)pp;
+				else
+					bv[qb & 1][i] = a.bias_dtype == 3 ? *(const float*)pp
+					                : a.bias_dtype == 2 ? (float)*(const __bf16*)pp
+					                                    : (float)*(const _Float16*)pp;
+			}
+		};
+		// bias values of block qb that belong to slot j when the 16 of them are spread over a stage
+		auto load_bias_for_slot = [&](int qb, int j) __attribute__((always_inline)) {
+			if constexpr (BIAS) {
+				if constexpr (NSLOT >= 16) {
+					if (j % (NSLOT / 16) == 0) load_bias(qb, j / (NSLOT / 16));
+				} else {
+#pragma unroll
+					for (int e = 0; e < 16 / NSLOT; ++e) load_bias(qb, j * (16 / NSLOT) + e);
+				}
 			}
 		};
 		auto mfma_A = [&](int qb, int j, f32x16& sa, f32x16& dpa) __attribute__((always_inline)) {
@@ -335,7 +350,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 				for (int e = e0; e < e1; ++e) {
 					int i = 4 * q + e;
 					if constexpr (BIAS)
-						bx[q][e] = (__builtin_fmaf(sa[i], c1, bv[i]) - lse4[q][e]) * kLog2e;
+						bx[q][e] = (__builtin_fmaf(sa[i], c1, bv[qb & 1][i]) - lse4[q][e]) * kLog2e;
 					else
 						bx[q][e] = __builtin_fmaf(sa[i], c1, -lse4[q][e]);
 				}
@@ -414,10 +429,6 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 						if constexpr (NSLOT >= 16) {
 							if (j % (NSLOT / 16) == NSLOT / 16 - 1) {
 								int ms = j / (NSLOT / 16);
-								if constexpr (BIAS) {
-									if (ms % 4 == 0)
-										for (int e = e0; e < e1; ++e) load_bias(k - 1, ms + e);
-								}
 								micro_B(k - 1, ms / 4, ms % 4, e0, e1, s[(k - 1) & 1], dp[(k - 1) & 1], pbits[(k - 1) & 1], sbits[(k - 1) & 1]);
 							}
 						} else {
@@ -427,15 +438,13 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 #pragma unroll
 							for (int e = 0; e < QPS; ++e) {
 								int q = grp * QPS + e;
-								if constexpr (BIAS) {
-									if (phase == 0)
-										for (int z = e0; z < e1; ++z) load_bias(k - 1, 4 * q + z);
-								}
 								micro_B(k - 1, q, phase, e0, e1, s[(k - 1) & 1], dp[(k - 1) & 1], pbits[(k - 1) & 1], sbits[(k - 1) & 1]);
 							}
 						}
 					}
 				};
+				// bias of the block whose elementwise stage comes next
+				if constexpr (NEXT_B) load_bias_for_slot(k, j);
 				if constexpr (HAS_A) mfma_A(k, j, s[k & 1], dp[k & 1]);
 				// the vector-ALU work below must not move above the product: for the products
 				// issued as inline assembly that order is what keeps a read of S / dP at least
@@ -870,7 +879,10 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 	if (a.stages & 2) {
 		a.mtiles = (a.Sk + C::KV_BN - 1) / C::KV_BN;
 		dim3 grid((unsigned)(a.mtiles * a.B * a.Hkv)), block(C::KV_NW * 64);
-		hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, C::KV_NW, C::KV_QB, BIAS, DROP>), grid, block, 0, s, a);
+		if (BIAS && a.bias_dtype == (std::is_same<T, BF16>::value ? 2 : 1))
+			hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, C::KV_NW, C::KV_QB, BIAS, DROP, BIAS>), grid, block, 0, s, a);
+		else
+			hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, C::KV_NW, C::KV_QB, BIAS, DROP, false>), grid, block, 0, s, a);
 	}
 	if (a.stages & 4) {
 		a.mtiles = (a.Sq + C::DQ_BM - 1) / C::DQ_BM;
