@@ -71,6 +71,10 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	// S / dP accumulators in VGPRs) when the AGPR file holds the former; the bias and dropout
 	// variants need the registers for other things and leave the choice to the compiler.
 	constexpr bool KV_AGPR = 2 * KS * 4 + 2 * DB * 16 <= 256 && !BIAS && !DROP;
+	// On that path the elementwise stage is shortened: K is pre-multiplied by scale * log2(e)
+	// and the chains of S and dP start from -lse and -delta instead of 0, so that
+	// P = exp2(S accumulator) and dS = P * (dP accumulator) need no further arithmetic.
+	constexpr bool FOLD = KV_AGPR;
 
 	// Q[0] Q[1] dO[0] dO[1] | lse[0] lse[1] delta[0] delta[1]
 	__shared__ __attribute__((aligned(1024))) char smem[4 * TILE_BYTES + 4 * STAT_BYTES];
@@ -125,6 +129,16 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		}
 	}
 
+	if constexpr (FOLD) {
+		const float kc = a.scale * kLog2e;
+#pragma unroll
+		for (int ks = 0; ks < KS; ++ks) {
+			typename T::V8 x = kf[ks];
+			kf[ks] = pack8<T>((float)x[0] * kc, (float)x[1] * kc, (float)x[2] * kc, (float)x[3] * kc, (float)x[4] * kc,
+			                  (float)x[5] * kc, (float)x[6] * kc, (float)x[7] * kc);
+		}
+	}
+
 	f32x16 dk[DB], dv[DB];
 #pragma unroll
 	for (int db = 0; db < DB; ++db)
@@ -172,6 +186,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 			} else {
 				x = a.delta[idx];
 			}
+			if constexpr (FOLD) x = -x;
 		}
 		return x;
 	};
@@ -287,10 +302,12 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		auto mfma_A = [&](int qb, int j, f32x16& sa, f32x16& dpa) __attribute__((always_inline)) {
 			int ks = j >> 1, r = (qb * NSLOT + j) % RING;
 			if constexpr (KV_AGPR) {
+				// the chains start from -lse and -delta of the block's rows (accumulator element i
+				// belongs to row 8 (i / 4) + 4 g + i % 4, which is element i % 4 of quarter i / 4)
 				if (j == 0)
-					mfma32_vz<true>(sa, afr[r], kf[ks]);
+					mfma32_vc(sa, afr[r], kf[ks], __builtin_shufflevector(__builtin_shufflevector(lse4[0], lse4[1], 0, 1, 2, 3, 4, 5, 6, 7), __builtin_shufflevector(lse4[2], lse4[3], 0, 1, 2, 3, 4, 5, 6, 7), 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15));
 				else if (j == 1)
-					mfma32_vz<true>(dpa, afr[r], vf[ks]);
+					mfma32_vc(dpa, afr[r], vf[ks], __builtin_shufflevector(__builtin_shufflevector(del4[0], del4[1], 0, 1, 2, 3, 4, 5, 6, 7), __builtin_shufflevector(del4[2], del4[3], 0, 1, 2, 3, 4, 5, 6, 7), 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15));
 				else if (j & 1)
 					mfma32_va<true>(dpa, afr[r], vf[ks]);
 				else
@@ -345,7 +362,31 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		};
 		auto micro_B = [&](int qb, int q, int phase, int e0, int e1, const f32x16& sa, const f32x16& dpa, u32x4(&pbo)[2], u32x4(&sbo)[2])
 		                   __attribute__((always_inline)) {
-			if (phase == 0) {
+			if constexpr (FOLD) {
+				// the accumulators already hold S scale log2(e) - lse and dP - delta
+				if (phase == 0) {
+#pragma unroll
+					for (int e = e0; e < e1; ++e) {
+						float p = exp2_fast(sa[4 * q + e]);
+						if constexpr (MASKED) {
+							int row = m0 + 32 * qb + 8 * q + 4 * g + e;
+							bool ok = row < sq_eff && jcol < sk_eff && (!a.causal || jcol <= row + off);
+							p = ok ? p : 0.f;
+						}
+						bx[q][e] = p;
+					}
+				} else if (phase == 2) {
+#pragma unroll
+					for (int e = e0; e < e1; ++e) by[q][e] = bx[q][e] * dpa[4 * q + e];
+				} else if (phase == 3) {
+					int hf = q >> 1, m = (q & 1) * 2;
+#pragma unroll
+					for (int e = e0; e < e1; e += 2) {
+						pbo[hf][m + e / 2] = pack2<typename T::V2>(bx[q][e], bx[q][e + 1]);
+						sbo[hf][m + e / 2] = pack2<typename T::V2>(by[q][e], by[q][e + 1]);
+					}
+				}
+			} else if (phase == 0) {
 #pragma unroll
 				for (int e = e0; e < e1; ++e) {
 					int i = 4 * q + e;
@@ -395,6 +436,10 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		// reads that the first PA slots of stage 0 use
 #pragma unroll
 		for (int j = 0; j < PA; ++j) issue_A(0, j);
+		if constexpr (FOLD) {
+#pragma unroll
+			for (int aa = 0; aa < 4; ++aa) issue_stat(0, aa);
+		}
 
 		auto stage = [&](auto k_tag) __attribute__((always_inline)) {
 			constexpr int k = decltype(k_tag)::value;
@@ -409,16 +454,20 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 					if (jn < NSLOT) {
 						if constexpr (HAS_A) issue_A(k, jn);
 						if constexpr (HAS_C) issue_C(k - 2, jn);
-						if constexpr (HAS_B) {
+						if constexpr (HAS_B && !FOLD) {
 							issue_stat_for_slot(k - 1, jn);
 						}
 					} else {
 						int jj = jn - NSLOT;
 						if constexpr (NEXT_A) issue_A(k + 1, jj);
 						if constexpr (NEXT_C) issue_C(k - 1, jj);
-						if constexpr (NEXT_B) {
+						if constexpr (NEXT_B && !FOLD) {
 							issue_stat_for_slot(k, jj);
 						}
+					}
+					// the start values of the chains of the next block, in the last four slots
+					if constexpr (FOLD && NEXT_A) {
+						if (j >= NSLOT - 4) issue_stat(k + 1, j - (NSLOT - 4));
 					}
 				}
 				// first half of the slot: product of A, first half of the micro-step(s) of B;
