@@ -108,7 +108,10 @@ int fa2_bwd(const fa2_params* p, void* hip_stream);
  * bit 0 = delta pre-pass (`_attn_bwd_preprocess`, _backward_triton.py:79-147),
  * bit 1 = dK/dV kernel (`_attn_bwd_block_dkdv`, :257-435),
  * bit 2 = dQ kernel (`_attn_bwd_block_dq`, :519-709).  fa2_bwd == stages 7.
- * The dK/dV and dQ kernels read the delta the pre-pass left in scratch. */
+ * With fewer than all three bits the dK/dV and dQ kernels read the delta an
+ * earlier pre-pass left in scratch.  With all three the pre-pass is not
+ * launched on its own: the dQ kernel forms delta from the O and dO rows it
+ * holds, leaves it in scratch and runs before the dK/dV kernel. */
 int fa2_bwd_stages(const fa2_params* p, void* hip_stream, int stages);
 
 /* Bytes of scratch fa2_bwd needs for these dimensions (0 on invalid params). */

@@ -721,6 +721,28 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 			}
 		}
 	}
+	// Whole backward in one call: delta = rowsum(O * dO) of the lane's row is formed here from
+	// the dO fragments already in registers (each half-wave holds half of the row) and left
+	// in scratch for the dK/dV kernel, which is launched after this one; the separate
+	// pre-pass (`_attn_bwd_preprocess`, _backward_triton.py:79-147) is then not launched.
+	if (a.dq_makes_delta) {
+		const char* obase_ = a.o.ptr + (int64_t)b * a.o.sb + (int64_t)h * a.o.sh;
+#pragma unroll
+		for (int qb = 0; qb < QB; ++qb) {
+			int i = qrow[qb] < a.Sq ? qrow[qb] : a.Sq - 1;
+			const char* op_ = obase_ + (int64_t)i * a.o.ss + g * 16;
+			float acc4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+			for (int ks = 0; ks < KS; ++ks) {
+				V8 ov = *(const V8*)(op_ + ks * 32);
+#pragma unroll
+				for (int e = 0; e < 8; ++e) acc4[e & 3] += (float)ov[e] * (float)dof[qb][ks][e];
+			}
+			float d = pair_sum((acc4[0] + acc4[1]) + (acc4[2] + acc4[3]));
+			del_r[qb] = d;
+			if (g == 0 && qrow[qb] < a.Sq) a.delta[((int64_t)b * a.Hq + h) * a.Sq + qrow[qb]] = d;
+		}
+	}
 
 	f32x16 dq[QB][DB];
 #pragma unroll
@@ -920,11 +942,22 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 	typedef BwdCfg<T, D> C;
 	int groups = a.B * a.Hkv;
 	a.xcd_remap = (groups % 8 == 0) ? 1 : 0;
-	if (a.stages & 1) {
+	// All three stages requested: the dQ kernel forms delta itself and runs first, the dK/dV
+	// kernel reads the delta it left in scratch.  Otherwise (per-kernel timing) each stage
+	// is launched as asked and the dQ / dK/dV kernels read the delta of an earlier pre-pass.
+	const bool fused_delta = (a.stages & 7) == 7;
+	a.dq_makes_delta = fused_delta ? 1 : 0;
+	if ((a.stages & 1) && !fused_delta) {
 		int64_t nrows = (int64_t)a.B * a.Sq * a.Hq;
 		constexpr int RPB = 256 / (D / 8);
 		hipLaunchKernelGGL((bwd_delta_kernel<T, D>), dim3((unsigned)((nrows + RPB - 1) / RPB)), dim3(256), 0, s, a);
 	}
+	auto launch_dq = [&]() {
+		a.mtiles = (a.Sq + C::DQ_BM - 1) / C::DQ_BM;
+		dim3 grid((unsigned)(a.mtiles * a.B * a.Hq)), block(C::DQ_NW * 64);
+		hipLaunchKernelGGL((bwd_dq_kernel<T, D, C::DQ_NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP>), grid, block, 0, s, a);
+	};
+	if (fused_delta) launch_dq();
 	if (a.stages & 2) {
 		a.mtiles = (a.Sk + C::KV_BN - 1) / C::KV_BN;
 		dim3 grid((unsigned)(a.mtiles * a.B * a.Hkv)), block(C::KV_NW * 64);
@@ -933,11 +966,7 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 		else
 			hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, C::KV_NW, C::KV_QB, BIAS, DROP, false>), grid, block, 0, s, a);
 	}
-	if (a.stages & 4) {
-		a.mtiles = (a.Sq + C::DQ_BM - 1) / C::DQ_BM;
-		dim3 grid((unsigned)(a.mtiles * a.B * a.Hq)), block(C::DQ_NW * 64);
-		hipLaunchKernelGGL((bwd_dq_kernel<T, D, C::DQ_NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP>), grid, block, 0, s, a);
-	}
+	if ((a.stages & 4) && !fused_delta) launch_dq();
 	return hipGetLastError();
 }
 

@@ -30,6 +30,7 @@ struct KArgs {
 	int mtiles;      // number of row tiles of the launched kernel
 	int xcd_remap;   // 1: group-major placement of workgroups on the 8 XCDs
 	int stages;      // backward: bit 0 delta, bit 1 dK/dV, bit 2 dQ
+	int dq_makes_delta;  // the dQ kernel computes delta itself (and stores it for the dK/dV kernel)
 };
 
 // dtype: FA2_FP16 / FA2_BF16.  Return hipError_t of the launch.
