@@ -22,7 +22,7 @@ AVAILABLE_BACKENDS = tp.Literal["gpu", "tpu", "cpu"]
 
 
 class Backend(str, Enum):
-	"""Supported compute backends."""
+	"""Device family the arrays live on (values as in the reference, :74-79)."""
 
 	GPU = "gpu"
 	TPU = "tpu"
@@ -30,7 +30,7 @@ class Backend(str, Enum):
 
 
 class Platform(str, Enum):
-	"""Supported Flash Attention platforms."""
+	"""Kernel family; `HIP` is the one this package implements (others: :82-87)."""
 
 	TRITON = "triton"
 	PALLAS = "pallas"
@@ -58,7 +58,8 @@ def _detect_backend() -> str:
 
 @dataclass
 class AttentionConfig:
-	"""Configuration for Flash Attention computation."""
+	"""Field for field the reference's dataclass (:90-99).  The block sizes are kept
+	for source compatibility; the gfx950 kernels use fixed, measured tile shapes."""
 
 	blocksize_q: int = 128
 	blocksize_k: int = 128
@@ -74,13 +75,16 @@ class AttentionConfig:
 			self.platform = self._default_platform()
 
 	def _default_platform(self) -> Platform:
-		"""Determines the default platform based on the backend."""
-		platform_map = {
-			Backend.GPU: Platform.HIP,
-			Backend.CPU: Platform.JAX,
-			Backend.TPU: Platform.PALLAS,
-		}
-		return platform_map.get(self.backend)
+		return _DEFAULT_PLATFORM.get(self.backend)
+
+
+_DEFAULT_PLATFORM = {Backend.GPU: Platform.HIP, Backend.CPU: Platform.JAX, Backend.TPU: Platform.PALLAS}
+
+# (backend, platform) pairs the constructor accepts: the reference's list (:124-132) plus HIP on a GPU
+_ACCEPTED_PAIRS = frozenset(
+	[(Backend.GPU, pl) for pl in (Platform.HIP, Platform.TRITON, Platform.PALLAS, Platform.JAX)]
+	+ [(Backend.CPU, Platform.JAX), (Backend.TPU, Platform.JAX), (Backend.TPU, Platform.PALLAS)]
+)
 
 
 def _is_jax_array(x) -> bool:
@@ -88,29 +92,17 @@ def _is_jax_array(x) -> bool:
 
 
 class FlashAttention:
-	"""Flash Attention implementation with multiple backend support."""
+	"""The reference's operator object (:117-356): validates the configuration once,
+	then dispatches every call to the platform's kernels."""
 
 	def __init__(self, config: tp.Optional[AttentionConfig] = None):
 		self.config = config or AttentionConfig()
 		self._validate_config()
 
 	def _validate_config(self):
-		"""Validates the configuration settings."""
-		valid_combinations = {
-			(Backend.GPU, Platform.HIP),
-			(Backend.GPU, Platform.TRITON),
-			(Backend.GPU, Platform.PALLAS),
-			(Backend.GPU, Platform.JAX),
-			(Backend.CPU, Platform.JAX),
-			(Backend.TPU, Platform.JAX),
-			(Backend.TPU, Platform.PALLAS),
-		}
-
-		if (self.config.backend, self.config.platform) not in valid_combinations:
-			raise ValueError(
-				f"Invalid backend-platform combination: "
-				f"{self.config.backend}-{self.config.platform}"
-			)
+		pair = (self.config.backend, self.config.platform)
+		if pair not in _ACCEPTED_PAIRS:
+			raise ValueError(f"Invalid backend-platform combination: {pair[0]}-{pair[1]}")
 
 	@staticmethod
 	def repeat_kv_heads(key, value, num_reps: int):
@@ -127,19 +119,11 @@ class FlashAttention:
 		"""Processes attention bias based on head configuration.  A bias with one
 		entry per KV head is accepted as is (the reference repeats it to the query
 		heads, :161-164; the HIP kernels index it by h // r instead)."""
-		if bias is None:
-			return None
-
-		if bias.shape[1] == num_q_heads or bias.shape[1] == 1:
+		if bias is None or bias.shape[1] in (num_q_heads, 1, num_kv_heads):
 			return bias
-
-		elif bias.shape[1] == num_kv_heads:
-			return bias
-		else:
-			raise ValueError(
-				f"Incompatible bias shape. Got {bias.shape[1]} heads, "
-				f"expected {num_q_heads}, {num_kv_heads}, or 1"
-			)
+		raise ValueError(
+			f"Incompatible bias shape. Got {bias.shape[1]} heads, expected {num_q_heads}, {num_kv_heads}, or 1"
+		)
 
 	def __call__(
 		self,
@@ -153,20 +137,14 @@ class FlashAttention:
 		dropout_seed: tp.Optional[int] = None,
 		adjust_sharindgs: bool = False,
 	):
-		"""
-		Computes flash attention using the configured backend and platform.
-		query [B, Sq, Hq, D], key/value [B, Sk, Hkv, D]; returns [B, Sq, Hq, D].
-		"""
-		num_q_heads = query.shape[2]
-		num_kv_heads = key.shape[2]
-
+		"""query [B, Sq, Hq, D], key/value [B, Sk, Hkv, D] -> [B, Sq, Hq, D]
+		(signature and checks of the reference's `__call__`, :171-214)."""
+		num_q_heads, num_kv_heads = query.shape[2], key.shape[2]
 		if num_q_heads % num_kv_heads != 0:
 			raise ValueError(
-				f"Query heads ({num_q_heads}) must be divisible by "
-				f"key/value heads ({num_kv_heads})"
+				f"Query heads ({num_q_heads}) must be divisible by key/value heads ({num_kv_heads})"
 			)
-		if bias is not None:
-			bias = self._handle_bias(bias, num_q_heads, num_kv_heads)
+		bias = self._handle_bias(bias, num_q_heads, num_kv_heads)
 		kw = dict(
 			query=query,
 			key=key,
@@ -256,21 +234,8 @@ def create_flash_attention(
 	platform: tp.Optional[tp.Union[Platform, str]] = None,
 	**kwargs,
 ) -> FlashAttention:
-	"""
-	Factory function to create a FlashAttention instance with the specified configuration.
-
-	Args:
-	    backend: Compute backend to use (GPU, TPU, or CPU)
-	    platform: Platform to use (HIP; Triton / Pallas resolve to HIP on a GPU)
-	    **kwargs: Additional configuration parameters for AttentionConfig
-
-	Returns:
-	    Configured FlashAttention instance
-	"""
-	if isinstance(backend, str):
-		backend = Backend(backend)
-	if isinstance(platform, str):
-		platform = Platform(platform)
-
-	config = AttentionConfig(backend=backend, platform=platform, **kwargs)
-	return FlashAttention(config)
+	"""Shorthand of the reference (:359-381): strings or enum members for backend and
+	platform, remaining keywords go to `AttentionConfig`."""
+	backend = Backend(backend) if isinstance(backend, str) else backend
+	platform = Platform(platform) if isinstance(platform, str) else platform
+	return FlashAttention(AttentionConfig(backend=backend, platform=platform, **kwargs))
