@@ -64,7 +64,8 @@ typedef struct fa2_params {
 	int32_t B, Sq, Sk, Hq, Hkv, D;
 	int32_t causal;         /* bottom-right aligned: j <= i + Sk - Sq
 	                           (_forward_triton.py:127-132)                */
-	float scale;            /* softmax scale, applied to q.k^T; must be > 0 */
+	float scale;            /* softmax scale, applied to q.k^T; must be > 0.  The dK/dV kernel keeps scale*log2(e)*k in the
+	                           element type, so for fp16 inputs |k|*scale*1.4427 must stay below 65504 */
 	float p_drop;           /* dropout probability in [0,1)                */
 	uint64_t seed;          /* Philox key for the dropout keep-mask        */
 

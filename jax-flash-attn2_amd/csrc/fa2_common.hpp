@@ -279,7 +279,10 @@ FA2_DEV void tile_load_async(FA2_LDS char* tile, const char* gbase, int64_t stri
 // and strides too large for 32-bit offsets take the general path above.
 FA2_DEV void lds_dma16_so(uint32_t lane_off, const char* uniform_base, FA2_LDS char* wave_dst) {
 	uint32_t m = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)wave_dst);
-	asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(uniform_base), "s"(m)
+	// s_nop 3: with s_mov that makes 5 wait states between a v_readfirstlane that produced the
+	// base and the memory instruction reading it as an SGPR operand; the compiler pads such
+	// hazards for its own instructions but does not look inside inline assembly
+	asm volatile("s_mov_b32 m0, %2\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(uniform_base), "s"(m)
 	             : "m0");
 }
 
