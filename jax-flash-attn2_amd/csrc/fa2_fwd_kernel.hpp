@@ -178,10 +178,30 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 		}
 	}
 
+	// Without bias the score only feeds exp2: Q is pre-multiplied by scale * log2(e) and the
+	// chain of S starts from minus the row's running reference instead of 0 (nm16: the value
+	// repeated over the 16 accumulator registers, all of which belong to the lane's row), so
+	// that P = exp2(S accumulator) with no further arithmetic.
+	constexpr bool FOLD = !BIAS;
+	if constexpr (FOLD) {
+		const float qc = a.scale * kLog2e;
+#pragma unroll
+		for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+			for (int ks = 0; ks < KS; ++ks) {
+				V8 x = qf[qb][ks];
+				qf[qb][ks] = pack8<T>((float)x[0] * qc, (float)x[1] * qc, (float)x[2] * qc, (float)x[3] * qc, (float)x[4] * qc,
+				                      (float)x[5] * qc, (float)x[6] * qc, (float)x[7] * qc);
+			}
+	}
+	f32x16 nm16[QB];
+
 	f32x16 oacc[QB][DB];
 	float mrow[QB], lrow[QB];
 #pragma unroll
 	for (int qb = 0; qb < QB; ++qb) {
+#pragma unroll
+		for (int i = 0; i < 16; ++i) nm16[qb][i] = 0.f;
 		mrow[qb] = -INFINITY;
 		lrow[qb] = 0.f;
 #pragma unroll
@@ -250,7 +270,8 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 			for (int kb = 0; kb < KB; ++kb) {
 				V8 kf = *(const FA2_LDS V8*)(kt + koff[ks] + kb * (32 * D * 2));
 #pragma unroll
-				for (int qb = 0; qb < QB; ++qb) s[kb][qb] = mfma32(kf, qf[qb][ks], s[kb][qb]);
+				for (int qb = 0; qb < QB; ++qb)
+					s[kb][qb] = mfma32(kf, qf[qb][ks], (FOLD && ks == 0) ? nm16[qb] : s[kb][qb]);
 			}
 		// issue order: a few fragment reads ahead, then one read per product, so that the
 		// LDS latency is paid once per tile instead of once per product
@@ -309,32 +330,61 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 				}
 			float mx = __builtin_fmaxf(__builtin_fmaxf(mx4[0], mx4[1]), __builtin_fmaxf(mx4[2], mx4[3]));
 			mx = pair_max(mx);
-			// to the softmax domain (log2 units without bias, natural units with bias)
-			if constexpr (!BIAS) mx = mx * c1;  // c1 > 0 is checked by the launcher
-			const float slack = BIAS ? kRescaleSlack * kLn2 : kRescaleSlack;
-			if (__builtin_amdgcn_ballot_w64(mx > mrow[qb] + slack) != 0) {
-				float m_new = __builtin_fmaxf(mrow[qb], mx);
-				float m_use = m_new == -INFINITY ? 0.f : m_new;
-				float alpha = BIAS ? exp2_fast((mrow[qb] - m_use) * kLog2e) : exp2_fast(mrow[qb] - m_use);
-				mrow[qb] = m_new;
-				lrow[qb] *= alpha;
-#pragma unroll
-				for (int db = 0; db < DB; ++db)
-#pragma unroll
-					for (int i = 0; i < 16; ++i) oacc[qb][db][i] *= alpha;
-			}
-			const float m_use = mrow[qb] == -INFINITY ? 0.f : mrow[qb];
-			const float nm = BIAS ? -m_use * kLog2e : -m_use;
 			float ls4[4] = {0.f, 0.f, 0.f, 0.f};
+			if constexpr (FOLD) {
+				// the accumulators hold x - m (log2 units), mx is the largest of them
+				const bool fresh = mrow[qb] == -INFINITY;  // no key seen so far: any finite maximum becomes the reference
+				if (__builtin_amdgcn_ballot_w64(mx > kRescaleSlack || (fresh && mx > -INFINITY)) != 0) {
+					const float m_old = fresh ? 0.f : mrow[qb];
+					float m_new = __builtin_fmaxf(mrow[qb], m_old + mx);
+					const float m_use = m_new == -INFINITY ? 0.f : m_new;
+					const float shift = m_use - m_old;
+					const float alpha = fresh ? 1.f : exp2_fast(-shift);  // (fresh: l = 0 and O = 0)
+					mrow[qb] = m_new;
+					lrow[qb] *= alpha;
 #pragma unroll
-			for (int kb = 0; kb < KB; ++kb)
+					for (int db = 0; db < DB; ++db)
 #pragma unroll
-				for (int i = 0; i < 16; ++i) {
-					float p = BIAS ? exp2_fast(__builtin_fmaf(s[kb][qb][i] - m_use, kLog2e, 0.f))
-					               : exp2_fast(__builtin_fmaf(s[kb][qb][i], c1, nm));
-					ls4[i & 3] += p;
-					s[kb][qb][i] = p;
+						for (int i = 0; i < 16; ++i) oacc[qb][db][i] *= alpha;
+#pragma unroll
+					for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+						for (int i = 0; i < 16; ++i) s[kb][qb][i] -= shift;
+#pragma unroll
+					for (int i = 0; i < 16; ++i) nm16[qb][i] = -m_use;
 				}
+#pragma unroll
+				for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+					for (int i = 0; i < 16; ++i) {
+						float p = exp2_fast(s[kb][qb][i]);
+						ls4[i & 3] += p;
+						s[kb][qb][i] = p;
+					}
+			} else {
+				// natural units with bias
+				const float slack = kRescaleSlack * kLn2;
+				if (__builtin_amdgcn_ballot_w64(mx > mrow[qb] + slack) != 0) {
+					float m_new = __builtin_fmaxf(mrow[qb], mx);
+					float m_use = m_new == -INFINITY ? 0.f : m_new;
+					float alpha = exp2_fast((mrow[qb] - m_use) * kLog2e);
+					mrow[qb] = m_new;
+					lrow[qb] *= alpha;
+#pragma unroll
+					for (int db = 0; db < DB; ++db)
+#pragma unroll
+						for (int i = 0; i < 16; ++i) oacc[qb][db][i] *= alpha;
+				}
+				const float m_use = mrow[qb] == -INFINITY ? 0.f : mrow[qb];
+#pragma unroll
+				for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+					for (int i = 0; i < 16; ++i) {
+						float p = exp2_fast(__builtin_fmaf(s[kb][qb][i] - m_use, kLog2e, 0.f));
+						ls4[i & 3] += p;
+						s[kb][qb][i] = p;
+					}
+			}
 			lrow[qb] += (ls4[0] + ls4[1]) + (ls4[2] + ls4[3]);
 			if constexpr (DROP) {
 #pragma unroll
