@@ -94,6 +94,12 @@ void fill(const fa2_params* p, KArgs& a) {
 		               a.bias_sm % valign == 0)
 		                  ? 1
 		                  : 0;
+		// tiles of bias can be copied to LDS like K / V tiles: element type of q, 16-byte aligned
+		// rows, whole tiles of 64 keys, row stride within the 32-bit offsets of the tile copies
+		a.bias_lds = (p->bias_dtype == p->dtype && ((uintptr_t)p->bias % 16) == 0 && a.bias_sb % 16 == 0 && a.bias_sh % 16 == 0 &&
+		              a.bias_sm % 16 == 0 && a.bias_sm >= 0 && a.bias_sm <= 0x7fffffff / 256 && p->Sk % 64 == 0)
+		                 ? 1
+		                 : 0;
 	}
 	a.seqlens = p->seqlens;
 	a.B = p->B;

@@ -76,10 +76,17 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	// P = exp2(S accumulator) and dS = P * (dP accumulator) need no further arithmetic.
 	constexpr bool FOLD = KV_AGPR;
 
-	// Q[0] Q[1] dO[0] dO[1] | lse[0] lse[1] delta[0] delta[1]
-	__shared__ __attribute__((aligned(1024))) char smem[4 * TILE_BYTES + 4 * STAT_BYTES];
+	// A bias in the element type of q is streamed through LDS as tiles of BMQ rows x BN keys
+	// where LDS has the room (the launcher then guarantees 16-byte aligned rows and whole key
+	// tiles): fetched one key per lane from global memory, every value is a 2-byte load of its own.
+	constexpr bool BIAS_LDS = BIAS && BIAS_T && D == 64;  // D = 128: no room in LDS; D = 256: no registers to spare
+	constexpr int BIAS_BYTES = BIAS_LDS ? BMQ * BN * 2 : 0;
+	static_assert(BN == 128, "bias tiles use the 128-element row geometry");
+	// Q[0] Q[1] dO[0] dO[1] | lse[0] lse[1] delta[0] delta[1] | bias[0] bias[1]
+	__shared__ __attribute__((aligned(1024))) char smem[4 * TILE_BYTES + 4 * STAT_BYTES + 2 * BIAS_BYTES];
 	FA2_LDS char* lds = (FA2_LDS char*)smem;
 	FA2_LDS char* stat = lds + 4 * TILE_BYTES;
+	FA2_LDS char* lds_bias = lds + 4 * TILE_BYTES + 4 * STAT_BYTES;
 
 	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
 	const int g = lane >> 5, c = lane & 31;
@@ -91,7 +98,14 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		int id = blockIdx.x;
 		int per_group = a.mtiles;
 		int grp, within;
-		if (a.xcd_remap) {
+		if (a.xcd_remap == 2) {
+			// bias shared by the heads: one batch per XCD, the kv-heads of one key tile adjacent
+			int xcd = id & 7, j = id >> 3;
+			int per_batch = per_group * a.Hkv;
+			int rem = j % per_batch;
+			grp = ((j / per_batch) * 8 + xcd) * a.Hkv + rem % a.Hkv;
+			within = rem / a.Hkv;
+		} else if (a.xcd_remap) {
 			int xcd = id & 7, j = id >> 3;
 			grp = (j / per_group) * 8 + xcd;
 			within = j % per_group;
@@ -161,6 +175,8 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	TileLoader<D, BMQ, NT> qload, doload;
 	qload.init(a.q.ss, tid);
 	doload.init(a.dout.ss, tid);
+	TileLoader<128, BMQ, NT> bload;
+	if constexpr (BIAS_LDS) bload.init(a.bias_sm, tid);
 	// start the copies of streamed tile `step` (rows beyond Sq are fetched from the last valid row)
 	auto issue_tile = [&](int step, FA2_LDS char* qdst, FA2_LDS char* dodst) __attribute__((always_inline)) {
 		int hq = hk * r + step / nq;
@@ -170,6 +186,11 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		const char* db_ = a.dout.ptr + (int64_t)b * a.dout.sb + (int64_t)hq * a.dout.sh + (int64_t)m0 * a.dout.ss;
 		qload.load(qdst, qb_, a.q.ss, rows, tid);
 		doload.load(dodst, db_, a.dout.ss, rows, tid);
+		if constexpr (BIAS_LDS) {
+			int hb = a.bias_group ? hk : hq;
+			const char* bb_ = a.bias + (int64_t)b * a.bias_sb + (int64_t)hb * a.bias_sh + (int64_t)m0 * a.bias_sm + (int64_t)n0 * 2;
+			bload.load(lds_bias + (step & 1) * BIAS_BYTES, bb_, a.bias_sm, rows, tid);
+		}
 	};
 	// per-row statistics of a tile: thread t < BMQ fetches lse, t in [BMQ, 2 BMQ) fetches delta
 	auto fetch_stat = [&](int step) -> float {
@@ -214,6 +235,16 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		}
 	}
 
+	// bias tile (rows of 128 keys): this lane's 8-byte piece of rows 4 g + i16 / 4 (+ 8) at its wave's 32 keys
+	int boffq[2] = {0, 0};
+	if constexpr (BIAS_LDS) {
+		int i16 = lane & 15;
+		int trow = 4 * g + (i16 >> 2);
+		int col = 32 * w + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
+		boffq[0] = tile_off<128>(trow, col >> 3) + ((col & 4) << 1);
+		boffq[1] = tile_off<128>(trow + 8, col >> 3) + ((col & 4) << 1);
+	}
+
 	// One streamed tile of BMQ query rows of q-head hq.  MASKED = some (row, key)
 	// of this wave's 32 keys x BMQ rows is masked.
 	auto tile_body = [&](auto masked_tag, const FA2_LDS char* qt, const FA2_LDS char* dot, int buf, int hq, int m0)
@@ -247,7 +278,9 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		V8 afr[RING];                     // fragments of Q_i / dO_i for the products of A
 		u32x4 cfr[RING];                  // transposed fragments of dO_i / Q_i for the products of C
 		f32x4 lse4[4], del4[4];
-		float bv[2][BIAS ? 16 : 1];       // [block parity]: bias values, fetched one stage ahead of their use
+		float bv[2][BIAS && !BIAS_LDS ? 16 : 1];  // [block parity]: bias values, fetched one stage ahead of their use
+		u32x2 bvr[2][BIAS_LDS ? 4 : 1];           // the same from LDS: [block parity][quad], 4 values of 16 bits
+		const FA2_LDS char* bt = lds_bias + buf * BIAS_BYTES;
 
 		// fragment of product j of A(qb): even j -> Q (S), odd j -> dO (dP), k-step j / 2
 		auto issue_A = [&](int qb, int j) __attribute__((always_inline)) {
@@ -276,7 +309,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 			}
 		};
 		auto load_bias = [&](int qb, int i) __attribute__((always_inline)) {
-			if constexpr (BIAS) {
+			if constexpr (BIAS && !BIAS_LDS) {
 				int row = m0 + 32 * qb + 8 * (i >> 2) + 4 * g + (i & 3);
 				row = row < a.Sq ? row : a.Sq - 1;
 				const char* pp = bias_base + (int64_t)row * a.bias_sm;
@@ -290,7 +323,14 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		};
 		// bias values of block qb that belong to slot j when the 16 of them are spread over a stage
 		auto load_bias_for_slot = [&](int qb, int j) __attribute__((always_inline)) {
-			if constexpr (BIAS) {
+			if constexpr (BIAS_LDS) {
+				// quad j (rows 8 j + 4 g + e of the block, this lane's key): one transposed read
+				if (j < 4) {
+					typedef __attribute__((__vector_size__(4 * sizeof(short)))) short v4s;
+					v4s x = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FA2_LDS v4s*)(bt + boffq[j & 1] + (j >> 1) * (16 * 256) + qb * (32 * 256)));
+					bvr[qb & 1][j] = __builtin_bit_cast(u32x2, x);
+				}
+			} else if constexpr (BIAS) {
 				if constexpr (NSLOT >= 16) {
 					if (j % (NSLOT / 16) == 0) load_bias(qb, j / (NSLOT / 16));
 				} else {
@@ -391,7 +431,12 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 				for (int e = e0; e < e1; ++e) {
 					int i = 4 * q + e;
 					if constexpr (BIAS)
-						bx[q][e] = (__builtin_fmaf(sa[i], c1, bv[qb & 1][i]) - lse4[q][e]) * kLog2e;
+						if constexpr (BIAS_LDS) {
+							float bvl = (float)__builtin_bit_cast(typename T::V4, bvr[qb & 1][q])[e];
+							bx[q][e] = (__builtin_fmaf(sa[i], c1, bvl) - lse4[q][e]) * kLog2e;
+						} else {
+							bx[q][e] = (__builtin_fmaf(sa[i], c1, bv[qb & 1][i]) - lse4[q][e]) * kLog2e;
+						}
 					else
 						bx[q][e] = __builtin_fmaf(sa[i], c1, -lse4[q][e]);
 				}
@@ -631,7 +676,11 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 	constexpr int NT = NW * 64;
 	constexpr int TILE_BYTES = BN * D * 2;
 
-	__shared__ __attribute__((aligned(1024))) char smem[4 * TILE_BYTES];
+	// bias tiles through LDS as in the forward kernel
+	constexpr bool BIAS_LDS = BIAS && D <= 128;
+	constexpr int BIAS_BYTES = BIAS_LDS ? BM * BN * 2 : 0;
+	static_assert(BN == 64, "bias tiles use the 64-element row geometry");
+	__shared__ __attribute__((aligned(1024))) char smem[4 * TILE_BYTES + 2 * BIAS_BYTES];
 	FA2_LDS char* lds = (FA2_LDS char*)smem;
 
 	int mt, h, b;
@@ -758,6 +807,17 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 		int hb = a.bias_group ? hk : h;
 		bias_base = a.bias + (int64_t)b * a.bias_sb + (int64_t)hb * a.bias_sh;
 	}
+	const bool bias_lds = BIAS_LDS && a.bias_lds;
+	TileLoader<64, BM, NT> bload;
+	int brows = 0, boff_lane = 0, bkey16 = 0;
+	if constexpr (BIAS_LDS) {
+		brows = a.Sq - m0 < BM ? a.Sq - m0 : BM;
+		bload.init(a.bias_sm, tid, brows);
+		int row = w * (QB * 32) + c;
+		boff_lane = row * 128 + 8 * g;
+		bkey16 = swz<64>(row) << 4;
+		if (bias_lds && ntiles > 0) bload.load(lds + 4 * TILE_BYTES, bias_base + (int64_t)m0 * a.bias_sm, a.bias_sm, brows, tid);
+	}
 
 	int koff[KS];
 #pragma unroll
@@ -775,12 +835,19 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 		}
 	}
 
-	auto tile_body = [&](auto masked_tag, const FA2_LDS char* kt, const FA2_LDS char* vt, int n0) {
+	auto tile_body = [&](auto masked_tag, const FA2_LDS char* kt, const FA2_LDS char* vt, const FA2_LDS char* bt, int n0) {
 		constexpr bool MASKED = decltype(masked_tag)::value;
 #pragma unroll
 		for (int kb = 0; kb < KB; ++kb) {
 			f32x4 bv[BIAS ? QB : 1][4];
-			if constexpr (BIAS) {
+			if (BIAS_LDS && bias_lds) {
+				static_assert(!BIAS_LDS || QB == 1, "");
+#pragma unroll
+				for (int aa = 0; aa < 4; ++aa) {
+					typename T::V4 x = *(const FA2_LDS typename T::V4*)(bt + boff_lane + (((kb * 4 + aa) << 4) ^ bkey16));
+					bv[0][aa] = __builtin_convertvector(x, f32x4);
+				}
+			} else if constexpr (BIAS) {
 #pragma unroll
 				for (int qb = 0; qb < QB; ++qb) {
 					int i = qrow[qb] < a.Sq ? qrow[qb] : a.Sq - 1;
@@ -887,13 +954,18 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 				    int rows = sk_eff - n1 < BN ? sk_eff - n1 : BN;
 				    kload.load(nk, kbase + (int64_t)n1 * a.k.ss, a.k.ss, rows, tid);
 				    vload.load(nv, vbase + (int64_t)n1 * a.v.ss, a.v.ss, rows, tid);
+				    if constexpr (BIAS_LDS) {
+					    if (bias_lds)
+						    bload.load(lds + 4 * TILE_BYTES + (buf ^ 1) * BIAS_BYTES, bias_base + (int64_t)m0 * a.bias_sm + (int64_t)n1 * 2,
+						               a.bias_sm, brows, tid);
+				    }
 			    }
 		    },
 		    [&](const FA2_LDS char* kt, const FA2_LDS char* vt) {
 			    if constexpr (decltype(masked_tag)::value) {
 				    if (n0 > wave_jmax) return;  // whole tile masked for this wave (uniform)
 			    }
-			    tile_body(masked_tag, kt, vt, n0);
+			    tile_body(masked_tag, kt, vt, lds + 4 * TILE_BYTES + buf * BIAS_BYTES, n0);
 		    });
 	};
 	// Tiles that lie entirely below every row's last allowed key need no mask.  They
@@ -942,6 +1014,7 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 	typedef BwdCfg<T, D> C;
 	int groups = a.B * a.Hkv;
 	a.xcd_remap = (groups % 8 == 0) ? 1 : 0;
+	if (BIAS && a.bias_sh == 0 && a.B % 8 == 0) a.xcd_remap = 2;
 	// All three stages requested: the dQ kernel forms delta itself and runs first, the dK/dV
 	// kernel reads the delta it left in scratch.  Otherwise (per-kernel timing) each stage
 	// is launched as asked and the dQ / dK/dV kernels read the delta of an earlier pre-pass.
@@ -961,7 +1034,11 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 	if (a.stages & 2) {
 		a.mtiles = (a.Sk + C::KV_BN - 1) / C::KV_BN;
 		dim3 grid((unsigned)(a.mtiles * a.B * a.Hkv)), block(C::KV_NW * 64);
-		if (BIAS && a.bias_dtype == (std::is_same<T, BF16>::value ? 2 : 1))
+		// typed variant: bias in the element type of q; where it stages the bias through LDS (D = 64)
+		// it also needs 16-byte aligned rows and whole tiles of 128 keys
+		bool typed = BIAS && a.bias_dtype == (std::is_same<T, BF16>::value ? 2 : 1);
+		if (D == 64 && !(a.bias_lds && a.Sk % C::KV_BN == 0)) typed = false;
+		if (typed)
 			hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, C::KV_NW, C::KV_QB, BIAS, DROP, BIAS>), grid, block, 0, s, a);
 		else
 			hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, C::KV_NW, C::KV_QB, BIAS, DROP, false>), grid, block, 0, s, a);

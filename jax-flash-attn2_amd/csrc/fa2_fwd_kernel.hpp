@@ -32,6 +32,18 @@ constexpr float kRescaleSlack = 8.f;
 // the longest, and starting them first shortens the tail of the launch.
 FA2_DEV void decode_block(const KArgs& a, int& mt, int& h, int& b) {
 	int id = blockIdx.x;
+	if (a.xcd_remap == 2) {
+		// A bias without a head axis is re-read by every head: one batch per XCD, and on an
+		// XCD the heads of one row tile next to each other, so that the tile of bias they all
+		// read is fetched into that XCD's L2 once.
+		int xcd = id & 7, j = id >> 3;
+		int per_batch = a.mtiles * a.Hq;
+		b = (j / per_batch) * 8 + xcd;
+		int rem = j % per_batch;
+		mt = a.mtiles - 1 - rem / a.Hq;
+		h = rem % a.Hq;
+		return;
+	}
 	int r = a.Hq / a.Hkv;
 	int per_group = a.mtiles * r;
 	int grp, within;
@@ -91,9 +103,14 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 	constexpr int NT = NW * 64;
 	constexpr int TILE_BYTES = BN * D * 2;
 
-	__shared__ __attribute__((aligned(1024))) char smem[4 * TILE_BYTES];
+	// Bias tiles (BM rows x 64 keys, element type of q) go through LDS as well when there is
+	// room: read from global memory one row per lane, a wave's load touches 32 cache lines.
+	constexpr bool BIAS_LDS = BIAS && D <= 128;
+	constexpr int BIAS_BYTES = BIAS_LDS ? BM * BN * 2 : 0;
+	static_assert(BN == 64, "bias tiles use the 64-element row geometry");
+	__shared__ __attribute__((aligned(1024))) char smem[4 * TILE_BYTES + 2 * BIAS_BYTES];
 	FA2_LDS char* lds = (FA2_LDS char*)smem;
-	// layout: K[0] K[1] V[0] V[1]
+	// layout: K[0] K[1] V[0] V[1] bias[0] bias[1]
 
 	int mt, h, b;
 	decode_block(a, mt, h, b);
@@ -216,6 +233,18 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 		int hb = a.bias_group ? hk : h;
 		bias_base = a.bias + (int64_t)b * a.bias_sb + (int64_t)hb * a.bias_sh;
 	}
+	const bool bias_lds = BIAS_LDS && a.bias_lds;
+	TileLoader<64, BM, NT> bload;
+	int brows = 0, boff_lane = 0, bkey16 = 0;
+	if constexpr (BIAS_LDS) {
+		brows = a.Sq - m0 < BM ? a.Sq - m0 : BM;
+		bload.init(a.bias_sm, tid, brows);
+		// this lane's row of the tile: byte offset of its chunk 0 (+ 8 bytes for the upper half-wave) and swizzle key
+		int row = w * (QB * 32) + c;
+		boff_lane = row * 128 + 8 * g;
+		bkey16 = swz<64>(row) << 4;
+		if (bias_lds && ntiles > 0) bload.load(lds + 4 * TILE_BYTES, bias_base + (int64_t)m0 * a.bias_sm, a.bias_sm, brows, tid);
+	}
 
 	// Per-lane LDS byte offsets with the swizzle folded in, so that every fragment
 	// read in the loop is base + register + immediate.
@@ -238,11 +267,20 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 	}
 
 	// One K/V tile.  MASKED = some element of the tile is masked for this wave.
-	auto tile_body = [&](auto masked_tag, const FA2_LDS char* kt, const FA2_LDS char* vt, int n0) {
+	auto tile_body = [&](auto masked_tag, const FA2_LDS char* kt, const FA2_LDS char* vt, const FA2_LDS char* bt, int n0) {
 		constexpr bool MASKED = decltype(masked_tag)::value;
 		// bias tile, fetched ahead of the matrix products
 		f32x4 bv[BIAS ? KB : 1][BIAS ? QB : 1][4];
-		if constexpr (BIAS) {
+		if (BIAS_LDS && bias_lds) {
+			static_assert(!BIAS_LDS || QB == 1, "");
+#pragma unroll
+			for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+				for (int aa = 0; aa < 4; ++aa) {
+					typename T::V4 x = *(const FA2_LDS typename T::V4*)(bt + boff_lane + (((kb * 4 + aa) << 4) ^ bkey16));
+					bv[kb][0][aa] = __builtin_convertvector(x, f32x4);
+				}
+		} else if constexpr (BIAS) {
 #pragma unroll
 			for (int qb = 0; qb < QB; ++qb) {
 				int i = qrow[qb] < a.Sq ? qrow[qb] : a.Sq - 1;
@@ -441,13 +479,18 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 				    int rows = sk_eff - n1 < BN ? sk_eff - n1 : BN;
 				    kload.load(nk, kbase + (int64_t)n1 * a.k.ss, a.k.ss, rows, tid);
 				    vload.load(nv, vbase + (int64_t)n1 * a.v.ss, a.v.ss, rows, tid);
+				    if constexpr (BIAS_LDS) {
+					    if (bias_lds)
+						    bload.load(lds + 4 * TILE_BYTES + (buf ^ 1) * BIAS_BYTES, bias_base + (int64_t)m0 * a.bias_sm + (int64_t)n1 * 2,
+						               a.bias_sm, brows, tid);
+				    }
 			    }
 		    },
 		    [&](const FA2_LDS char* kt, const FA2_LDS char* vt) {
 			    if constexpr (decltype(masked_tag)::value) {
 				    if (n0 > wave_jmax) return;  // whole tile masked for this wave (uniform)
 			    }
-			    tile_body(masked_tag, kt, vt, n0);
+			    tile_body(masked_tag, kt, vt, lds + 4 * TILE_BYTES + buf * BIAS_BYTES, n0);
 		    });
 	};
 	// Tiles that lie entirely below every row's last allowed key need no mask.  They
@@ -505,6 +548,7 @@ hipError_t launch_fwd_t(bool bias, bool drop, KArgs& a, hipStream_t s) {
 	a.mtiles = (a.Sq + C::BM - 1) / C::BM;
 	int groups = a.B * a.Hkv;
 	a.xcd_remap = (groups % 8 == 0) ? 1 : 0;
+	if (bias && a.bias_sh == 0 && a.B % 8 == 0) a.xcd_remap = 2;
 	dim3 grid((unsigned)(a.mtiles * a.B * a.Hq)), block(C::NW * 64);
 	if (bias && drop)
 		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, C::WPS, true, true>), grid, block, 0, s, a);

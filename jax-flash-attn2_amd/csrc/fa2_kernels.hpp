@@ -21,6 +21,7 @@ struct KArgs {
 	int bias_dtype;  // FA2_FP16 / FA2_BF16 / FA2_FP32
 	int bias_group;  // head axis of bias indexed by kv-head
 	int bias_vec4;   // rows are 4-element aligned: vector loads allowed
+	int bias_lds;    // bias tiles may be copied global->LDS in 16-byte pieces (see fa2_api.hip)
 	const int32_t* seqlens;
 	int B, Sq, Sk, Hq, Hkv;
 	int causal;
@@ -29,6 +30,7 @@ struct KArgs {
 	float drop_inv_keep;
 	int mtiles;      // number of row tiles of the launched kernel
 	int xcd_remap;   // 1: group-major placement of workgroups on the 8 XCDs
+	                 // 2: batch-major placement, heads of a row tile adjacent (a bias shared by the heads stays in L2)
 	int stages;      // backward: bit 0 delta, bit 1 dK/dV, bit 2 dQ
 	int dq_makes_delta;  // the dQ kernel computes delta itself (and stores it for the dK/dV kernel)
 };
