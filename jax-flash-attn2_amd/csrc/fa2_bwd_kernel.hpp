@@ -388,16 +388,38 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		// dropout keep bits of a quad (bit e = value 4q + e), produced one value per slot while
 		// the previous quad is processed: one Philox call at a time keeps its registers few
 		uint32_t keepw[4] = {0u, 0u, 0u, 0u};
-		auto keep_bit = [&](int qb, int q, int e) __attribute__((always_inline)) {
+		// One generator call yields the words of 4 adjacent keys of one row, and the 4 lanes of a
+		// quad hold 4 adjacent keys: lane t of a quad evaluates row e = t of the quad of rows,
+		// reduces its 4 words to 4 keep bits, and the quad exchanges them (DPP broadcasts).  The
+		// call is cut into 4 parts (rounds 0-2, 3-5, 6-7, 8-9 + exchange) that run in the four
+		// micro-step slots of the previous quad.  `u` selects one of two calls in flight.
+		uint32_t phs[2][4];
+		auto keep_bit = [&](int qb, int q, int part, int u = 0) __attribute__((always_inline)) {
 			if constexpr (DROP) {
-				int row = m0 + 32 * qb + 8 * q + 4 * g + e;
-				u32x4 rnd = philox4x32_10((uint32_t)(jcol >> 2), (uint32_t)row, (uint32_t)hq, (uint32_t)b, a.drop_k0, a.drop_k1);
-				uint32_t word = rnd[0];
-				word = (jcol & 3) == 1 ? rnd[1] : word;
-				word = (jcol & 3) == 2 ? rnd[2] : word;
-				word = (jcol & 3) == 3 ? rnd[3] : word;
-				uint32_t bit = word >= a.drop_thr ? (1u << e) : 0u;
-				keepw[q & 3] = e == 0 ? bit : (keepw[q & 3] | bit);
+				uint32_t(&cs)[4] = phs[u];
+				if (part == 0) {
+					cs[0] = (uint32_t)(jcol >> 2);
+					cs[1] = (uint32_t)(m0 + 32 * qb + 8 * q + 4 * g + (c & 3));
+					cs[2] = (uint32_t)hq;
+					cs[3] = (uint32_t)b;
+					philox4x32_rounds<0, 3>(cs, a.drop_k0, a.drop_k1);
+				} else if (part == 1) {
+					philox4x32_rounds<3, 6>(cs, a.drop_k0, a.drop_k1);
+				} else if (part == 2) {
+					philox4x32_rounds<6, 8>(cs, a.drop_k0, a.drop_k1);
+				} else {
+					philox4x32_rounds<8, 10>(cs, a.drop_k0, a.drop_k1);
+					// bit t = key (jcol & ~3) + t of this lane's row is kept
+					uint32_t mine = (cs[0] >= a.drop_thr ? 1u : 0u) | (cs[1] >= a.drop_thr ? 2u : 0u) | (cs[2] >= a.drop_thr ? 4u : 0u) |
+					                (cs[3] >= a.drop_thr ? 8u : 0u);
+					// row e was evaluated by lane e of the quad; this lane's key is bit c & 3 of its mask
+					uint32_t r0 = (uint32_t)__builtin_amdgcn_mov_dpp((int)mine, 0x00, 0xf, 0xf, false);
+					uint32_t r1 = (uint32_t)__builtin_amdgcn_mov_dpp((int)mine, 0x55, 0xf, 0xf, false);
+					uint32_t r2 = (uint32_t)__builtin_amdgcn_mov_dpp((int)mine, 0xaa, 0xf, 0xf, false);
+					uint32_t r3 = (uint32_t)__builtin_amdgcn_mov_dpp((int)mine, 0xff, 0xf, 0xf, false);
+					const uint32_t sh = (uint32_t)(c & 3);
+					keepw[q & 3] = ((r0 >> sh) & 1u) | (((r1 >> sh) & 1u) << 1) | (((r2 >> sh) & 1u) << 2) | (((r3 >> sh) & 1u) << 3);
+				}
 			}
 		};
 		auto micro_B = [&](int qb, int q, int phase, int e0, int e1, const f32x16& sa, const f32x16& dpa, u32x4(&pbo)[2], u32x4(&sbo)[2])
@@ -558,7 +580,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 						constexpr int QPS = 16 / NSLOT;
 						for (int e = 0; e < QPS; ++e) {
 							int q = (j / 4) * QPS + e;
-							if (q + QPS < 4) keep_bit(k - 1, q + QPS, j % 4);
+							if (q + QPS < 4) keep_bit(k - 1, q + QPS, j % 4, e);
 						}
 					}
 				}
@@ -569,7 +591,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 							keep_bit(k, 0, (j - (NSLOT - 4 * (NSLOT / 16))) / (NSLOT / 16));
 					} else {
 						if (j >= NSLOT - 4)
-							for (int e = 0; e < 16 / NSLOT; ++e) keep_bit(k, e, j - (NSLOT - 4));
+							for (int e = 0; e < 16 / NSLOT; ++e) keep_bit(k, e, j - (NSLOT - 4), e);
 					}
 				}
 				__builtin_amdgcn_sched_barrier(0);

@@ -355,6 +355,23 @@ FA2_DEV u32x4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, 
 	return out;
 }
 
+// Rounds [R0, R1) of the same generator on a counter kept by the caller, for callers that
+// spread one evaluation over several places of their instruction stream.
+template <int R0, int R1>
+FA2_DEV void philox4x32_rounds(uint32_t (&c)[4], uint32_t k0, uint32_t k1) {
+#pragma unroll
+	for (int r = R0; r < R1; ++r) {
+		uint32_t kr0 = k0 + (uint32_t)r * 0x9E3779B9u, kr1 = k1 + (uint32_t)r * 0xBB67AE85u;
+		uint32_t hi0 = __umulhi(0xD2511F53u, c[0]), lo0 = 0xD2511F53u * c[0];
+		uint32_t hi1 = __umulhi(0xCD9E8D57u, c[2]), lo1 = 0xCD9E8D57u * c[2];
+		uint32_t n0 = hi1 ^ c[1] ^ kr0, n2 = hi0 ^ c[3] ^ kr1;
+		c[0] = n0;
+		c[1] = lo1;
+		c[2] = n2;
+		c[3] = lo0;
+	}
+}
+
 struct Dropout {
 	uint32_t k0, k1, thr;
 	float inv_keep;  // 1 / (1 - p)
