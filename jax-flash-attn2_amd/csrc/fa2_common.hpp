@@ -341,8 +341,11 @@ FA2_DEV void wait_async_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"
 FA2_DEV u32x4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1) {
 #pragma unroll
 	for (int r = 0; r < 10; ++r) {
-		uint32_t hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
-		uint32_t hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+		// written as one 32 x 32 -> 64 bit product each (one v_mad_u64_u32 instead of a high and a low multiply)
+		uint64_t p0 = (uint64_t)0xD2511F53u * (uint64_t)c0;
+		uint64_t p1 = (uint64_t)0xCD9E8D57u * (uint64_t)c2;
+		uint32_t hi0 = (uint32_t)(p0 >> 32), lo0 = (uint32_t)p0;
+		uint32_t hi1 = (uint32_t)(p1 >> 32), lo1 = (uint32_t)p1;
 		uint32_t n0 = hi1 ^ c1 ^ k0, n2 = hi0 ^ c3 ^ k1;
 		c0 = n0;
 		c1 = lo1;
@@ -362,8 +365,11 @@ FA2_DEV void philox4x32_rounds(uint32_t (&c)[4], uint32_t k0, uint32_t k1) {
 #pragma unroll
 	for (int r = R0; r < R1; ++r) {
 		uint32_t kr0 = k0 + (uint32_t)r * 0x9E3779B9u, kr1 = k1 + (uint32_t)r * 0xBB67AE85u;
-		uint32_t hi0 = __umulhi(0xD2511F53u, c[0]), lo0 = 0xD2511F53u * c[0];
-		uint32_t hi1 = __umulhi(0xCD9E8D57u, c[2]), lo1 = 0xCD9E8D57u * c[2];
+		// written as one 32 x 32 -> 64 bit product each
+		uint64_t p0 = (uint64_t)0xD2511F53u * (uint64_t)c[0];
+		uint64_t p1 = (uint64_t)0xCD9E8D57u * (uint64_t)c[2];
+		uint32_t hi0 = (uint32_t)(p0 >> 32), lo0 = (uint32_t)p0;
+		uint32_t hi1 = (uint32_t)(p1 >> 32), lo1 = (uint32_t)p1;
 		uint32_t n0 = hi1 ^ c[1] ^ kr0, n2 = hi0 ^ c[3] ^ kr1;
 		c[0] = n0;
 		c[1] = lo1;
