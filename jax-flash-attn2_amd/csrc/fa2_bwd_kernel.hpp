@@ -822,6 +822,14 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 		for (int db = 0; db < DB; ++db)
 #pragma unroll
 			for (int i = 0; i < 16; ++i) dq[qb][db][i] = 0.f;
+	// Without dropout the chain of dP starts from -delta of the lane's row (the 16 accumulator
+	// registers all belong to that row), so dS = P * (dP accumulator) without a subtraction.
+	constexpr bool FOLD_DP = !DROP && !BIAS && D <= 128;  // (the other variants have no registers to spare)
+	f32x16 ndel16[QB];
+#pragma unroll
+	for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+		for (int i = 0; i < 16; ++i) ndel16[qb][i] = -del_r[qb];
 
 	const float c1 = BIAS ? a.scale : a.scale * kLog2e;
 	const char* bias_base = nullptr;
@@ -892,7 +900,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 				for (int qb = 0; qb < QB; ++qb) s[qb] = mfma32(ka, qf[qb][ks], s[qb]);
 				V8 va = *(const FA2_LDS V8*)(vt + koff[ks] + kb * (32 * D * 2));
 #pragma unroll
-				for (int qb = 0; qb < QB; ++qb) dp[qb] = mfma32(va, dof[qb][ks], dp[qb]);
+				for (int qb = 0; qb < QB; ++qb) dp[qb] = mfma32(va, dof[qb][ks], (FOLD_DP && ks == 0) ? ndel16[qb] : dp[qb]);
 			}
 			// issue order: a few fragment reads ahead, then one read per product
 			{
@@ -940,7 +948,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 						}
 						float dpe = dp[qb][i];
 						if constexpr (DROP) dpe = rnd[e] >= a.drop_thr ? dpe * a.drop_inv_keep : 0.f;
-						s[qb][i] = p * (dpe - del_r[qb]);
+						s[qb][i] = FOLD_DP ? p * dpe : p * (dpe - del_r[qb]);
 					}
 				}
 #pragma unroll
