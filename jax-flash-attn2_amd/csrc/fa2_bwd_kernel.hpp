@@ -79,7 +79,8 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	// A bias in the element type of q is streamed through LDS as tiles of BMQ rows x BN keys
 	// where LDS has the room (the launcher then guarantees 16-byte aligned rows and whole key
 	// tiles): fetched one key per lane from global memory, every value is a 2-byte load of its own.
-	constexpr bool BIAS_LDS = BIAS && BIAS_T && D == 64;  // D = 128: no room in LDS; D = 256: no registers to spare
+	// (D = 128: LDS has room only with 64-row tiles, which the launcher chooses for bias; D = 256: no registers to spare)
+	constexpr bool BIAS_LDS = BIAS && BIAS_T && 4 * TILE_BYTES + 4 * STAT_BYTES + 2 * BMQ * BN * 2 <= 160 * 1024 && D <= 128;
 	constexpr int BIAS_BYTES = BIAS_LDS ? BMQ * BN * 2 : 0;
 	static_assert(BN == 128, "bias tiles use the 128-element row geometry");
 	// Q[0] Q[1] dO[0] dO[1] | lse[0] lse[1] delta[0] delta[1] | bias[0] bias[1]
@@ -1064,14 +1065,16 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 	if (a.stages & 2) {
 		a.mtiles = (a.Sk + C::KV_BN - 1) / C::KV_BN;
 		dim3 grid((unsigned)(a.mtiles * a.B * a.Hkv)), block(C::KV_NW * 64);
-		// typed variant: bias in the element type of q; where it stages the bias through LDS (D = 64)
+		// typed variant: bias in the element type of q; where it stages the bias through LDS (D <= 128)
 		// it also needs 16-byte aligned rows and whole tiles of 128 keys
 		bool typed = BIAS && a.bias_dtype == (std::is_same<T, BF16>::value ? 2 : 1);
-		if (D == 64 && !(a.bias_lds && a.Sk % C::KV_BN == 0)) typed = false;
+		if (D <= 128 && !(a.bias_lds && a.Sk % C::KV_BN == 0)) typed = false;
+		// with bias at D = 128 the streamed tiles are 64 rows, which leaves LDS room for the bias tiles
+		constexpr int QBV = (BIAS && D == 128) ? 2 : C::KV_QB;
 		if (typed)
-			hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, C::KV_NW, C::KV_QB, BIAS, DROP, BIAS>), grid, block, 0, s, a);
+			hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, C::KV_NW, QBV, BIAS, DROP, BIAS>), grid, block, 0, s, a);
 		else
-			hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, C::KV_NW, C::KV_QB, BIAS, DROP, false>), grid, block, 0, s, a);
+			hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, C::KV_NW, QBV, BIAS, DROP, false>), grid, block, 0, s, a);
 	}
 	if ((a.stages & 4) && !fused_delta) launch_dq();
 	return hipGetLastError();
