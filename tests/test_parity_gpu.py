@@ -74,6 +74,17 @@ def test_bias_broadcast(bshape, D):
 	_run_case(B, Sq, Sk, Hq, Hkv, D, torch.bfloat16, causal=True, bias_shape=(*bshape, Sq, Sk), data_seed=3)
 
 
+@pytest.mark.parametrize("bshape", [(1, 1), (2, 1), (2, 4), (2, 2)], ids=["b1h1", "bBh1", "bBhH", "bBhKV"])
+@pytest.mark.parametrize("D", [64, 128])
+def test_bias_whole_key_tiles(bshape, D):
+	"""Sk a multiple of 128 with a bias in the element type of q: the kernels copy bias tiles to
+	LDS instead of loading single values (ragged query rows, causal and not, dropout on top)."""
+	B, Sq, Sk, Hq, Hkv = 2, 200, 256, 4, 2
+	_run_case(B, Sq, Sk, Hq, Hkv, D, torch.bfloat16, causal=False, bias_shape=(*bshape, Sq, Sk))
+	_run_case(B, Sq, Sk, Hq, Hkv, D, torch.float16, causal=True, bias_shape=(*bshape, Sq, Sk), data_seed=5)
+	_run_case(B, 256, 256, Hq, Hkv, D, torch.bfloat16, causal=True, bias_shape=(*bshape, 256, 256), p=0.2, seed=11, data_seed=6)
+
+
 def test_bias_dtypes_and_unaligned_rows():
 	# fp32 bias with a 16-bit q; odd Sk makes bias rows unaligned for vector loads
 	_run_case(1, 70, 75, 2, 2, 64, torch.float16, bias_shape=(1, 2, 70, 75), bias_dtype=torch.float32)
