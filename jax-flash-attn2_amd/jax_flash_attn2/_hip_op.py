@@ -41,6 +41,24 @@ def _t4(x: torch.Tensor) -> Fa2Tensor:
 	return t
 
 
+# Head dims the kernels are built for.  Any other head dim up to 256 is zero-padded to the next
+# one, as the reference pads to the next power of two (_forward_triton.py:525-526): zero
+# columns of q / k leave the scores unchanged, zero columns of v and dO give zero columns of
+# O, dV and dQ / dK, which are cut off again.  The softmax scale keeps using the true head dim.
+HEAD_DIMS = (64, 128, 256)
+
+
+def _kernel_head_dim(D: int) -> int:
+	for d in HEAD_DIMS:
+		if D <= d:
+			return d
+	raise ValueError(f"head dim {D} is not supported (at most {HEAD_DIMS[-1]})")
+
+
+def _pad_d(x: torch.Tensor, Dp: int) -> torch.Tensor:
+	return x if x.shape[-1] == Dp else torch.nn.functional.pad(x, (0, Dp - x.shape[-1]))
+
+
 def _usable(x: torch.Tensor) -> torch.Tensor:
 	"""Kernels read 16 bytes at a time along D: unit D stride, 16-byte aligned rows."""
 	if x.stride(3) != 1 or any(s % 8 for s in x.stride()[:3]) or x.data_ptr() % 16:
@@ -96,10 +114,12 @@ def _seqlens_from_mask(attention_mask, q):
 def fwd(q, k, v, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, causal=False, dropout_seed=None):
 	"""Returns (out [B,Sq,Hq,D] in q.dtype, lse [B,Hq,Sq] fp32 natural log)."""
 	lib = _lib.load()
-	q, k, v = _usable(q), _usable(k), _usable(v)
+	D0 = q.shape[-1]
+	D = _kernel_head_dim(D0)
+	q, k, v = _usable(_pad_d(q, D)), _usable(_pad_d(k, D)), _usable(_pad_d(v, D))
 	bias = _prep_bias(bias)
-	B, Sq, Hq, D = q.shape
-	scale = 1.0 / math.sqrt(D) if softmax_scale is None else softmax_scale
+	B, Sq, Hq, _ = q.shape
+	scale = 1.0 / math.sqrt(D0) if softmax_scale is None else softmax_scale
 	out = torch.empty((B, Sq, Hq, D), dtype=q.dtype, device=q.device)
 	lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
 	p = _lib.new_params()
@@ -107,17 +127,19 @@ def fwd(q, k, v, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, 
 	p.o = _t4(out)
 	p.lse = lse.data_ptr()
 	_lib.check(lib.fa2_fwd(ctypes.byref(p), _stream_ptr(q.device)))
-	return out, lse
+	return (out if D == D0 else out[..., :D0]), lse
 
 
 def bwd(q, k, v, out, lse, dout, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, causal=False,
         dropout_seed=None):
 	"""Returns (dq, dk, dv) in the dtypes of q, k, v; dk/dv summed over each KV group."""
 	lib = _lib.load()
-	q, k, v, out, dout = _usable(q), _usable(k), _usable(v), _usable(out), _usable(dout)
+	D0 = q.shape[-1]
+	D = _kernel_head_dim(D0)
+	q, k, v, out, dout = (_usable(_pad_d(x, D)) for x in (q, k, v, out, dout))
 	bias = _prep_bias(bias)
-	B, Sq, Hq, D = q.shape
-	scale = 1.0 / math.sqrt(D) if softmax_scale is None else softmax_scale
+	B, Sq, Hq, _ = q.shape
+	scale = 1.0 / math.sqrt(D0) if softmax_scale is None else softmax_scale
 	dq = torch.empty_like(q, memory_format=torch.contiguous_format)
 	dk = torch.empty_like(k, memory_format=torch.contiguous_format)
 	dv = torch.empty_like(v, memory_format=torch.contiguous_format)
@@ -131,6 +153,8 @@ def bwd(q, k, v, out, lse, dout, bias=None, seqlens=None, softmax_scale=None, dr
 	p.scratch = scratch.data_ptr()
 	p.scratch_bytes = scratch.numel()
 	_lib.check(lib.fa2_bwd(ctypes.byref(p), _stream_ptr(q.device)))
+	if D != D0:
+		dq, dk, dv = dq[..., :D0], dk[..., :D0], dv[..., :D0]
 	return dq, dk, dv
 
 

@@ -81,3 +81,15 @@ def test_unbuilt_platforms_say_so():
 		create_flash_attention("cpu", "jax")(q, q, q)
 	with pytest.raises(NotImplementedError):
 		create_flash_attention("tpu", "pallas")(q, q, q)
+
+
+def test_kernel_head_dim_padding_rule():
+	torch = pytest.importorskip("torch")
+	from jax_flash_attn2 import _hip_op
+
+	assert [_hip_op._kernel_head_dim(d) for d in (16, 64, 65, 128, 129, 256)] == [64, 64, 128, 128, 256, 256]
+	with pytest.raises(ValueError):
+		_hip_op._kernel_head_dim(257)
+	x = torch.ones(1, 2, 3, 80)
+	y = _hip_op._pad_d(x, 128)
+	assert y.shape == (1, 2, 3, 128) and float(y[..., 80:].abs().sum()) == 0.0 and _hip_op._pad_d(y, 128) is y

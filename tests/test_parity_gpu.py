@@ -74,6 +74,14 @@ def test_bias_broadcast(bshape, D):
 	_run_case(B, Sq, Sk, Hq, Hkv, D, torch.bfloat16, causal=True, bias_shape=(*bshape, Sq, Sk), data_seed=3)
 
 
+@pytest.mark.parametrize("D", [32, 80, 96, 160, 192])
+def test_other_head_dims(D):
+	"""Head dims between the built ones are zero-padded by the host layer (the reference pads
+	to the next power of two, _forward_triton.py:525-526); scale stays 1/sqrt(D)."""
+	_run_case(2, 150, 150, 4, 2, D, torch.bfloat16, causal=True)
+	_run_case(1, 96, 130, 2, 2, D, torch.float16, causal=False, bias_shape=(1, 2, 96, 130), data_seed=4)
+
+
 @pytest.mark.parametrize("bshape", [(1, 1), (2, 1), (2, 4), (2, 2)], ids=["b1h1", "bBh1", "bBhH", "bBhKV"])
 @pytest.mark.parametrize("D", [64, 128])
 def test_bias_whole_key_tiles(bshape, D):
