@@ -137,8 +137,8 @@ def cpu_baseline(w):
 def main():
 	ap = argparse.ArgumentParser()
 	ap.add_argument("--gpus", type=int, default=1)
-	ap.add_argument("--steps", type=int, default=20)
-	ap.add_argument("--warmup", type=int, default=3)
+	ap.add_argument("--steps", type=int, default=50)
+	ap.add_argument("--warmup", type=int, default=5)
 	ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
 	ap.add_argument("--no-cpu-baseline", action="store_true")
 	ap.add_argument("--copy-calibration", action="store_true",
@@ -175,6 +175,14 @@ def main():
 			dst.copy_(src)
 		torch.cuda.synchronize()
 		del src, dst
+
+	# Untimed pre-roll: after idling the GPU needs some hundred milliseconds of work before its
+	# clocks settle (the first steps after start-up run 10-15 % slower than the steady state).
+	t_pre = time.perf_counter()
+	while time.perf_counter() - t_pre < 0.5:
+		for _ in range(5):
+			step()
+		torch.cuda.synchronize()
 
 	for _ in range(args.warmup):
 		step()

@@ -92,13 +92,22 @@ typedef struct fa2_params {
 	/* Backward only. */
 	fa2_tensor dout;        /* dO, read                                    */
 	fa2_tensor dq, dk, dv;  /* written; dk/dv already summed over each KV group */
-	void* scratch;          /* >= fa2_bwd_scratch_bytes(p) bytes, 256-byte aligned */
+	/* Backward: required, >= fa2_bwd_scratch_bytes(p) bytes.  Forward: optional, see
+	 * fa2_fwd_scratch_bytes().  256-byte aligned. */
+	void* scratch;
 	uint64_t scratch_bytes;
 } fa2_params;
 
 /* O = softmax(scale q k^T + bias, masked) v, with dropout; writes o and lse.
  * Replaces the `_attn_fwd` custom call (_forward_triton.py:547-588). */
 int fa2_fwd(const fa2_params* p, void* hip_stream);
+
+/* Optional scratch for fa2_fwd.  Non-zero for a short query (Sq <= 64) over many keys with
+ * too few (batch, head) pairs to fill the chip - decoding, `Sq == 1` in
+ * flash_attention.py:239-242: given `scratch` (256-byte aligned) of at least this many
+ * bytes, fa2_fwd splits the keys into ranges handled by separate workgroups and merges the
+ * partial results (same O and lse to rounding).  Without it the call runs unsplit. */
+size_t fa2_fwd_scratch_bytes(const fa2_params* p);
 
 /* dq, dk, dv from (q, k, v, o, lse, dO).  Replaces the `_attn_bwd_preprocess`
  * and `_attn_bwd` custom calls and the XLA reduce over the KV group

@@ -155,11 +155,46 @@ size_t fa2_bwd_scratch_bytes(const fa2_params* p) {
 	return (n + 255) & ~(size_t)255;
 }
 
+// Key ranges for a split forward: few query rows (one row tile of 64), too few (batch, head)
+// pairs to fill the chip, many keys.  Returns the number of ranges (1 = no split).
+static int fwd_split_plan(const fa2_params* p, int* split_len) {
+	*split_len = 0;
+	if (p->Sq > 64) return 1;
+	long base = (long)p->B * p->Hq;
+	int tiles = (p->Sk + 63) / 64;
+	if (base >= 512 || tiles < 8) return 1;
+	long want = (1024 + base - 1) / base;
+	if (want > tiles / 4) want = tiles / 4;
+	if (want > 64) want = 64;
+	if (want < 2) return 1;
+	int per = (int)((tiles + want - 1) / want);
+	*split_len = per * 64;
+	return (tiles + per - 1) / per;
+}
+
+size_t fa2_fwd_scratch_bytes(const fa2_params* p) {
+	if (!p || p->struct_size < sizeof(fa2_params)) return 0;
+	if (p->B <= 0 || p->Hq <= 0 || p->Sq <= 0 || p->Sk <= 0 || p->D <= 0) return 0;
+	int len;
+	int n = fwd_split_plan(p, &len);
+	if (n <= 1) return 0;
+	size_t rows = (size_t)n * (size_t)p->B * (size_t)p->Hq * (size_t)p->Sq;
+	return (rows * ((size_t)p->D + 1) * sizeof(float) + 255) & ~(size_t)255;
+}
+
 int fa2_fwd(const fa2_params* p, void* hip_stream) {
 	int rc = validate(p, 0);
 	if (rc) return rc;
 	KArgs a;
 	fill(p, a);
+	// optional scratch: with enough of it a short query over many keys runs split over key ranges
+	size_t need = fa2_fwd_scratch_bytes(p);
+	if (need && p->scratch && ((uintptr_t)p->scratch & 255) == 0 && p->scratch_bytes >= need) {
+		a.nsplit = fwd_split_plan(p, &a.split_len);
+		size_t rows = (size_t)a.nsplit * (size_t)p->B * (size_t)p->Hq * (size_t)p->Sq;
+		a.o_part = (float*)p->scratch;
+		a.lse_part = a.o_part + rows * (size_t)p->D;
+	}
 	hipError_t e = fa2::launch_fwd(p->dtype, p->D, p->bias != nullptr, p->p_drop > 0.f, a, (hipStream_t)hip_stream);
 	return e == hipSuccess ? FA2_OK : FA2_EHIP;
 }

@@ -30,8 +30,7 @@ constexpr float kRescaleSlack = 8.f;
 // fetched from HBM once per XCD L2 instead of once per L2 of every XCD.
 // Row tiles are visited last-first: under a causal mask the last tiles are
 // the longest, and starting them first shortens the tail of the launch.
-FA2_DEV void decode_block(const KArgs& a, int& mt, int& h, int& b) {
-	int id = blockIdx.x;
+FA2_DEV void decode_block(const KArgs& a, int& mt, int& h, int& b, int id = (int)blockIdx.x) {
 	if (a.xcd_remap == 2) {
 		// A bias without a head axis is re-read by every head: one batch per XCD, and on an
 		// XCD the heads of one row tile next to each other, so that the tile of bias they all
@@ -92,7 +91,12 @@ FA2_DEV f32x4 load_bias4(const char* rowp, int col, int dtype, bool vec_ok, int 
 	return out;
 }
 
-template <typename T, int D, int NW, int QB, int WPS, bool BIAS, bool DROP>
+// SPLIT: the keys are cut into a.nsplit ranges of a.split_len keys (a multiple of the tile);
+// workgroup (tile, split) handles one range and leaves a normalised partial result (O as
+// fp32 and its logsumexp) in scratch for fwd_combine_kernel.  For few query rows and many
+// keys (decoding, short cross-attention queries), where one workgroup per row tile would
+// leave most of the chip idle.
+template <typename T, int D, int NW, int QB, int WPS, bool BIAS, bool DROP, bool SPLIT = false>
 __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 	typedef typename T::V8 V8;
 	constexpr int BM = NW * QB * 32;
@@ -112,8 +116,13 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 	FA2_LDS char* lds = (FA2_LDS char*)smem;
 	// layout: K[0] K[1] V[0] V[1] bias[0] bias[1]
 
-	int mt, h, b;
-	decode_block(a, mt, h, b);
+	int mt, h, b, split = 0;
+	if constexpr (SPLIT) {
+		split = (int)blockIdx.x % a.nsplit;
+		decode_block(a, mt, h, b, (int)blockIdx.x / a.nsplit);
+	} else {
+		decode_block(a, mt, h, b);
+	}
 	const int hk = h / (a.Hq / a.Hkv);
 	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
 	const int g = lane >> 5, c = lane & 31;
@@ -129,7 +138,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 	const int m0 = mt * BM;
 	const int wm0 = m0 + w * (QB * 32);
 
-	// keys this row tile can see
+	// keys this row tile can see (of this workgroup's range of keys)
 	int kv_end = sk_eff;
 	if (a.causal) {
 		int last_row = (m0 + BM - 1 < sq_eff - 1) ? m0 + BM - 1 : sq_eff - 1;
@@ -137,7 +146,15 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 		kv_end = e < kv_end ? e : kv_end;
 	}
 	if (m0 >= sq_eff) kv_end = 0;
-	const int ntiles = kv_end > 0 ? (kv_end + BN - 1) / BN : 0;
+	int t_begin = 0;
+	if constexpr (SPLIT) {
+		int kv_begin = split * a.split_len;  // a multiple of BN
+		int e = kv_begin + a.split_len;
+		kv_end = e < kv_end ? e : kv_end;
+		t_begin = kv_begin / BN;
+		if (kv_end <= kv_begin) kv_end = 0;
+	}
+	const int ntiles = kv_end > 0 ? (kv_end + BN - 1) / BN : 0;  // one past the last tile
 
 	// per-lane last allowed key for each of this lane's rows
 	int jmax[QB];
@@ -176,10 +193,11 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 	kload.init(a.k.ss, tid);
 	vload.init(a.v.ss, tid);
 	// prologue: first K/V tile in flight while Q is fetched
-	if (ntiles > 0) {
-		int rows = sk_eff < BN ? sk_eff : BN;
-		kload.load(lds, kbase, a.k.ss, rows, tid);
-		vload.load(lds + 2 * TILE_BYTES, vbase, a.v.ss, rows, tid);
+	if (ntiles > t_begin) {
+		int nb = t_begin * BN, bsel = t_begin & 1;
+		int rows = sk_eff - nb < BN ? sk_eff - nb : BN;
+		kload.load(lds + bsel * TILE_BYTES, kbase + (int64_t)nb * a.k.ss, a.k.ss, rows, tid);
+		vload.load(lds + (2 + bsel) * TILE_BYTES, vbase + (int64_t)nb * a.v.ss, a.v.ss, rows, tid);
 	}
 
 	// Q fragments (B operand of S^T): lane holds Q[row c][16ks + 8g .. +7]
@@ -243,7 +261,9 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 		int row = w * (QB * 32) + c;
 		boff_lane = row * 128 + 8 * g;
 		bkey16 = swz<64>(row) << 4;
-		if (bias_lds && ntiles > 0) bload.load(lds + 4 * TILE_BYTES, bias_base + (int64_t)m0 * a.bias_sm, a.bias_sm, brows, tid);
+		if (bias_lds && ntiles > t_begin)
+			bload.load(lds + 4 * TILE_BYTES + (t_begin & 1) * BIAS_BYTES, bias_base + (int64_t)m0 * a.bias_sm + (int64_t)t_begin * BN * 2,
+			           a.bias_sm, brows, tid);
 	}
 
 	// Per-lane LDS byte offsets with the swizzle folded in, so that every fragment
@@ -497,8 +517,8 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 	// run in a loop of their own, so that the steady-state loop is a single
 	// straight-line body; the tiles on the causal diagonal / ragged end follow.
 	int t_full = (wave_jmin + 1) / BN;
-	t_full = t_full < 0 ? 0 : (t_full > ntiles ? ntiles : t_full);
-	for (int t = 0; t < t_full; ++t) step(std::false_type{}, t);
+	t_full = t_full < t_begin ? t_begin : (t_full > ntiles ? ntiles : t_full);
+	for (int t = t_begin; t < t_full; ++t) step(std::false_type{}, t);
 	for (int t = t_full; t < ntiles; ++t) step(std::true_type{}, t);
 
 	// epilogue: normalise, store O (lane: row c, four consecutive d per store) and LSE
@@ -509,6 +529,27 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 		float inv = lt > 0.f ? 1.f / lt : 0.f;
 		if constexpr (DROP) inv *= a.drop_inv_keep;
 		int i = qrow[qb];
+		if constexpr (SPLIT) {
+			// partial result of this key range: [split][b][h][i][D] fp32 and [split][b][h][i]
+			if (i < a.Sq) {
+				int64_t row = (((int64_t)split * a.B + b) * a.Hq + h) * a.Sq + i;
+				float* rp = a.o_part + row * D;
+#pragma unroll
+				for (int db = 0; db < DB; ++db)
+#pragma unroll
+					for (int aa = 0; aa < 4; ++aa) {
+						const f32x16& r = oacc[qb][db];
+						f32x4 o4 = {r[4 * aa] * inv, r[4 * aa + 1] * inv, r[4 * aa + 2] * inv, r[4 * aa + 3] * inv};
+						*(f32x4*)(rp + 32 * db + 8 * aa + 4 * g) = o4;
+					}
+				if (g == 0) {
+					float lse = -INFINITY;
+					if (lt > 0.f) lse = BIAS ? mrow[qb] + log2_fast(lt) * kLn2 : (mrow[qb] + log2_fast(lt)) * kLn2;
+					a.lse_part[row] = lse;
+				}
+			}
+			continue;
+		}
 		if (i < a.Sq) {
 			char* rp = obase + (int64_t)i * a.o.ss;
 #pragma unroll
@@ -532,6 +573,43 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 	}
 }
 
+// O = sum_s exp(lse_s - lse) O_s, lse = log sum_s exp(lse_s) over the key ranges of a split forward.
+// One thread per (row, 8 head-dim values); HBM-bound and small.
+template <typename T, int D>
+__global__ __launch_bounds__(256) void fwd_combine_kernel(const KArgs a) {
+	constexpr int TPR = D / 8;
+	constexpr int RPB = 256 / TPR;
+	int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / TPR;
+	int part = threadIdx.x % TPR;
+	int64_t nrows = (int64_t)a.B * a.Hq * a.Sq;
+	if (row >= nrows) return;
+	int i = (int)(row % a.Sq);
+	int64_t bh = row / a.Sq;
+	int h = (int)(bh % a.Hq), b = (int)(bh / a.Hq);
+	float m = -INFINITY;
+	for (int s = 0; s < a.nsplit; ++s) m = __builtin_fmaxf(m, a.lse_part[(int64_t)s * nrows + row]);
+	float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+	float tot = 0.f;
+	if (m > -INFINITY) {
+		for (int s = 0; s < a.nsplit; ++s) {
+			float wgt = exp2_fast((a.lse_part[(int64_t)s * nrows + row] - m) * kLog2e);
+			tot += wgt;
+			const float* op = a.o_part + ((int64_t)s * nrows + row) * D + part * 8;
+			f32x4 x0 = *(const f32x4*)op, x1 = *(const f32x4*)(op + 4);
+#pragma unroll
+			for (int e = 0; e < 4; ++e) {
+				acc[e] += wgt * x0[e];
+				acc[4 + e] += wgt * x1[e];
+			}
+		}
+	}
+	float inv = tot > 0.f ? 1.f / tot : 0.f;
+	char* rp = a.o.ptr + (int64_t)b * a.o.sb + (int64_t)h * a.o.sh + (int64_t)i * a.o.ss + part * 16;
+	*(typename T::V8*)rp = pack8<T>(acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv, acc[4] * inv, acc[5] * inv, acc[6] * inv,
+	                                acc[7] * inv);
+	if (part == 0) a.lse[row] = tot > 0.f ? m + log2_fast(tot) * kLn2 : -INFINITY;
+}
+
 template <typename T, int D>
 struct FwdCfg {
 	// D <= 128: 8 waves, two per SIMD (<= 256 registers each): while one waits on LDS or
@@ -542,8 +620,31 @@ struct FwdCfg {
 	static constexpr int BM = NW * QB * 32;
 };
 
+// Split forward: 2 waves x 32 rows per workgroup (the query is short), nsplit key ranges each.
+template <typename T, int D>
+hipError_t launch_fwd_split_t(bool bias, bool drop, KArgs& a, hipStream_t s) {
+	constexpr int NW = 2, BM = NW * 32;
+	a.mtiles = (a.Sq + BM - 1) / BM;
+	int groups = a.B * a.Hkv;
+	a.xcd_remap = (groups % 8 == 0) ? 1 : 0;
+	dim3 grid((unsigned)(a.mtiles * a.B * a.Hq * a.nsplit)), block(NW * 64);
+	if (bias && drop)
+		hipLaunchKernelGGL((fwd_kernel<T, D, NW, 1, 1, true, true, true>), grid, block, 0, s, a);
+	else if (bias)
+		hipLaunchKernelGGL((fwd_kernel<T, D, NW, 1, 1, true, false, true>), grid, block, 0, s, a);
+	else if (drop)
+		hipLaunchKernelGGL((fwd_kernel<T, D, NW, 1, 1, false, true, true>), grid, block, 0, s, a);
+	else
+		hipLaunchKernelGGL((fwd_kernel<T, D, NW, 1, 1, false, false, true>), grid, block, 0, s, a);
+	int64_t nrows = (int64_t)a.B * a.Hq * a.Sq;
+	constexpr int RPB = 256 / (D / 8);
+	hipLaunchKernelGGL((fwd_combine_kernel<T, D>), dim3((unsigned)((nrows + RPB - 1) / RPB)), dim3(256), 0, s, a);
+	return hipGetLastError();
+}
+
 template <typename T, int D>
 hipError_t launch_fwd_t(bool bias, bool drop, KArgs& a, hipStream_t s) {
+	if (a.nsplit > 1) return launch_fwd_split_t<T, D>(bias, drop, a, s);
 	typedef FwdCfg<T, D> C;
 	a.mtiles = (a.Sq + C::BM - 1) / C::BM;
 	int groups = a.B * a.Hkv;

@@ -33,6 +33,10 @@ struct KArgs {
 	                 // 2: batch-major placement, heads of a row tile adjacent (a bias shared by the heads stays in L2)
 	int stages;      // backward: bit 0 delta, bit 1 dK/dV, bit 2 dQ
 	int dq_makes_delta;  // the dQ kernel computes delta itself (and stores it for the dK/dV kernel)
+	// split forward (0 / 1 = off): key ranges of split_len keys, partial results in scratch
+	int nsplit, split_len;
+	float* o_part;    // [nsplit, B, Hq, Sq, D] fp32
+	float* lse_part;  // [nsplit, B, Hq, Sq] fp32
 };
 
 // dtype: FA2_FP16 / FA2_BF16.  Return hipError_t of the launch.

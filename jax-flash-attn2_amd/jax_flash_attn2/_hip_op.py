@@ -126,6 +126,12 @@ def fwd(q, k, v, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, 
 	_fill_common(p, q, k, v, bias, seqlens, scale, dropout_prob, causal, dropout_seed or 0)
 	p.o = _t4(out)
 	p.lse = lse.data_ptr()
+	# short query over many keys: scratch lets the library split the keys over workgroups
+	need = lib.fa2_fwd_scratch_bytes(ctypes.byref(p))
+	if need:
+		scratch = torch.empty((need,), dtype=torch.uint8, device=q.device)
+		p.scratch = scratch.data_ptr()
+		p.scratch_bytes = need
 	_lib.check(lib.fa2_fwd(ctypes.byref(p), _stream_ptr(q.device)))
 	return (out if D == D0 else out[..., :D0]), lse
 

@@ -65,6 +65,7 @@ EXPORTS = (
 	"fa2_bwd",
 	"fa2_bwd_stages",
 	"fa2_bwd_scratch_bytes",
+	"fa2_fwd_scratch_bytes",
 	"fa2_dropout_mask",
 	"fa2_validate",
 	"fa2_strerror",
@@ -104,6 +105,8 @@ def load() -> ctypes.CDLL:
 		lib.fa2_bwd_stages.restype = ctypes.c_int
 		lib.fa2_bwd_scratch_bytes.argtypes = [pp]
 		lib.fa2_bwd_scratch_bytes.restype = ctypes.c_size_t
+		lib.fa2_fwd_scratch_bytes.argtypes = [pp]
+		lib.fa2_fwd_scratch_bytes.restype = ctypes.c_size_t
 		lib.fa2_dropout_mask.argtypes = [pp, ctypes.c_void_p, ctypes.c_void_p]
 		lib.fa2_dropout_mask.restype = ctypes.c_int
 		lib.fa2_validate.argtypes = [pp, ctypes.c_int]

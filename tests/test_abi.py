@@ -130,3 +130,22 @@ def test_missing_library_fails_loudly(monkeypatch):
 	monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libfa2_hip.so")
 	with pytest.raises(ImportError):
 		_lib.load()
+
+
+def test_forward_scratch_only_for_short_queries_over_many_keys():
+	"""fa2_fwd_scratch_bytes: non-zero exactly where the split forward applies."""
+	lib = _lib.load()
+
+	def need(B, Sq, Sk, Hq, D=128):
+		p = _lib.new_params()
+		p.B, p.Sq, p.Sk, p.Hq, p.Hkv, p.D = B, Sq, Sk, Hq, Hq, D
+		return lib.fa2_fwd_scratch_bytes(ctypes.byref(p))
+
+	assert need(4, 4096, 4096, 32) == 0          # training shape: one pass
+	assert need(1, 1, 256, 8) == 0               # too few keys to split
+	assert need(64, 1, 8192, 32) == 0            # enough (batch, head) pairs already
+	n = need(1, 1, 8192, 8)
+	assert n > 0 and n % 256 == 0
+	# ranges x rows x (D values + logsumexp) floats, rounded up to 256 bytes
+	assert n >= 2 * 8 * (128 + 1) * 4 and n <= 64 * 8 * (128 + 1) * 4 + 256
+	assert need(1, 65, 8192, 8) == 0             # more than one row tile of 64

@@ -74,6 +74,33 @@ def test_bias_broadcast(bshape, D):
 	_run_case(B, Sq, Sk, Hq, Hkv, D, torch.bfloat16, causal=True, bias_shape=(*bshape, Sq, Sk), data_seed=3)
 
 
+@pytest.mark.parametrize(
+	"shape",
+	[
+		# B, Sq, Sk, Hq, Hkv, D, dtype, causal, bias heads, p
+		(1, 1, 4096, 8, 2, 128, torch.bfloat16, False, None, 0.0),
+		(2, 17, 1500, 4, 4, 64, torch.float16, True, None, 0.0),
+		(1, 64, 2048, 2, 1, 256, torch.bfloat16, True, 2, 0.1),
+		(2, 5, 1024, 4, 2, 128, torch.bfloat16, False, 1, 0.0),
+		(1, 33, 777, 2, 2, 64, torch.bfloat16, True, None, 0.25),
+	],
+	ids=["decode_gqa", "short_causal_fp16", "d256_bias_dropout", "bias_lds", "ragged_dropout"],
+)
+def test_short_query_split_over_keys(shape):
+	"""Sq <= 64 over many keys: the forward runs split over key ranges (partial results merged by
+	a second kernel) when the caller provides scratch, as the host layer does.  `Sq == 1` is the
+	decoding case of flash_attention.py:239-242."""
+	import ctypes
+
+	from jax_flash_attn2 import _lib
+
+	B, Sq, Sk, Hq, Hkv, D, dtype, causal, bh, p = shape
+	pr = _lib.new_params()
+	pr.B, pr.Sq, pr.Sk, pr.Hq, pr.Hkv, pr.D = B, Sq, Sk, Hq, Hkv, D
+	assert _lib.load().fa2_fwd_scratch_bytes(ctypes.byref(pr)) > 0, "this shape is meant to take the split path"
+	_run_case(B, Sq, Sk, Hq, Hkv, D, dtype, causal=causal, bias_shape=None if bh is None else (B, bh, Sq, Sk), p=p, seed=3)
+
+
 @pytest.mark.parametrize("D", [32, 80, 96, 160, 192])
 def test_other_head_dims(D):
 	"""Head dims between the built ones are zero-padded by the host layer (the reference pads
