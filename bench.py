@@ -107,8 +107,10 @@ def cpu_baseline(w):
 	import fa2_oracle as O
 
 	r = w["Hq"] // w["Hkv"]
-	B, S, D = 1, min(w["S"], 4096), w["D"]
-	Hkv = min(2, w["Hkv"])
+	# bounded sample: at most two batch entries and 4096 positions of the workload, all heads
+	# (10 - 20 s on 16 host cores for the workloads with S >= 4096)
+	B, S, D = min(w["B"], 2), min(w["S"], 4096), w["D"]
+	Hkv = w["Hkv"]
 	Hq = Hkv * r
 	rng = np.random.default_rng(0)
 	q = rng.standard_normal((B, S, Hq, D), dtype=np.float32) * 0.5
