@@ -157,10 +157,15 @@ size_t fa2_bwd_scratch_bytes(const fa2_params* p) {
 
 // Key ranges for a split forward: few query rows (one row tile of 64), too few (batch, head)
 // pairs to fill the chip, many keys.  Returns the number of ranges (1 = no split).
+// the rows of all q-heads of a kv-head fit one row tile: they share one workgroup (and one pass over K, V)
+static bool fwd_pack_gqa(const fa2_params* p) {
+	return p->Hkv > 0 && p->Hq % p->Hkv == 0 && p->Hq > p->Hkv && (long)(p->Hq / p->Hkv) * p->Sq <= 64;
+}
+
 static int fwd_split_plan(const fa2_params* p, int* split_len) {
 	*split_len = 0;
 	if (p->Sq > 64) return 1;
-	long base = (long)p->B * p->Hq;
+	long base = (long)p->B * (fwd_pack_gqa(p) ? p->Hkv : p->Hq);
 	int tiles = (p->Sk + 63) / 64;
 	if (base >= 512 || tiles < 8) return 1;
 	long want = (1024 + base - 1) / base;
@@ -191,6 +196,7 @@ int fa2_fwd(const fa2_params* p, void* hip_stream) {
 	size_t need = fa2_fwd_scratch_bytes(p);
 	if (need && p->scratch && ((uintptr_t)p->scratch & 255) == 0 && p->scratch_bytes >= need) {
 		a.nsplit = fwd_split_plan(p, &a.split_len);
+		a.pack_gqa = fwd_pack_gqa(p) ? 1 : 0;
 		size_t rows = (size_t)a.nsplit * (size_t)p->B * (size_t)p->Hq * (size_t)p->Sq;
 		a.o_part = (float*)p->scratch;
 		a.lse_part = a.o_part + rows * (size_t)p->D;

@@ -117,9 +117,21 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 	// layout: K[0] K[1] V[0] V[1] bias[0] bias[1]
 
 	int mt, h, b, split = 0;
+	// pack (split kernel only): the rows of the tile are the Sq rows of ALL r q-heads of one
+	// kv-head (row = head_in_group * Sq + position), so that K and V are streamed once per
+	// group instead of once per q-head; every lane then has its own q-head.
+	bool pack = false;
 	if constexpr (SPLIT) {
 		split = (int)blockIdx.x % a.nsplit;
-		decode_block(a, mt, h, b, (int)blockIdx.x / a.nsplit);
+		pack = a.pack_gqa != 0;
+		if (pack) {
+			int id2 = (int)blockIdx.x / a.nsplit;
+			b = id2 / a.Hkv;
+			h = (id2 % a.Hkv) * (a.Hq / a.Hkv);
+			mt = 0;
+		} else {
+			decode_block(a, mt, h, b, (int)blockIdx.x / a.nsplit);
+		}
 	} else {
 		decode_block(a, mt, h, b);
 	}
@@ -159,9 +171,21 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 	// per-lane last allowed key for each of this lane's rows
 	int jmax[QB];
 	int qrow[QB];
+	int hl[QB];  // this lane's q-head
 #pragma unroll
 	for (int qb = 0; qb < QB; ++qb) {
 		int i = wm0 + 32 * qb + c;
+		hl[qb] = h;
+		if (pack) {
+			int r = a.Hq / a.Hkv;
+			int hh = i / a.Sq;
+			i -= hh * a.Sq;
+			if (hh >= r) {  // beyond the group's rows: no such row
+				hh = r - 1;
+				i = a.Sq;
+			}
+			hl[qb] = h + hh;
+		}
 		qrow[qb] = i;
 		int jm = sk_eff - 1;
 		if (a.causal) jm = (i + off < jm) ? i + off : jm;
@@ -184,6 +208,10 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 			}
 			if (last >= sq_eff) wave_jmin = -1;
 		}
+		if (pack) {  // rows of several heads: every tile takes the masked path
+			wave_jmin = -1;
+			wave_jmax = wm0 < (a.Hq / a.Hkv) * a.Sq ? sk_eff - 1 : -1;
+		}
 	}
 
 	const char* kbase = a.k.ptr + (int64_t)b * a.k.sb + (int64_t)hk * a.k.sh;
@@ -203,9 +231,9 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 	// Q fragments (B operand of S^T): lane holds Q[row c][16ks + 8g .. +7]
 	V8 qf[QB][KS];
 	{
-		const char* qbase = a.q.ptr + (int64_t)b * a.q.sb + (int64_t)h * a.q.sh;
 #pragma unroll
 		for (int qb = 0; qb < QB; ++qb) {
+			const char* qbase = a.q.ptr + (int64_t)b * a.q.sb + (int64_t)hl[qb] * a.q.sh;
 			int i = qrow[qb] < a.Sq ? qrow[qb] : a.Sq - 1;
 			const char* rp = qbase + (int64_t)i * a.q.ss + g * 16;
 #pragma unroll
@@ -251,7 +279,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 		int hb = a.bias_group ? hk : h;
 		bias_base = a.bias + (int64_t)b * a.bias_sb + (int64_t)hb * a.bias_sh;
 	}
-	const bool bias_lds = BIAS_LDS && a.bias_lds;
+	const bool bias_lds = BIAS_LDS && a.bias_lds && !pack;
 	TileLoader<64, BM, NT> bload;
 	int brows = 0, boff_lane = 0, bkey16 = 0;
 	if constexpr (BIAS_LDS) {
@@ -305,6 +333,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 			for (int qb = 0; qb < QB; ++qb) {
 				int i = qrow[qb] < a.Sq ? qrow[qb] : a.Sq - 1;
 				const char* rowp = bias_base + (int64_t)i * a.bias_sm;
+				if (SPLIT && !a.bias_group) rowp += (int64_t)(hl[qb] - h) * a.bias_sh;  // (packed rows: the lane's own head)
 #pragma unroll
 				for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
@@ -450,7 +479,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 #pragma unroll
 					for (int aa = 0; aa < 4; ++aa) {
 						int j4 = (n0 + 32 * kb + 8 * aa + 4 * g) >> 2;
-						u32x4 rnd = philox4x32_10((uint32_t)j4, (uint32_t)qrow[qb], (uint32_t)h, (uint32_t)b, a.drop_k0, a.drop_k1);
+						u32x4 rnd = philox4x32_10((uint32_t)j4, (uint32_t)qrow[qb], (uint32_t)hl[qb], (uint32_t)b, a.drop_k0, a.drop_k1);
 #pragma unroll
 						for (int e = 0; e < 4; ++e)
 							s[kb][qb][4 * aa + e] = rnd[e] >= a.drop_thr ? s[kb][qb][4 * aa + e] : 0.f;
@@ -532,7 +561,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 		if constexpr (SPLIT) {
 			// partial result of this key range: [split][b][h][i][D] fp32 and [split][b][h][i]
 			if (i < a.Sq) {
-				int64_t row = (((int64_t)split * a.B + b) * a.Hq + h) * a.Sq + i;
+				int64_t row = (((int64_t)split * a.B + b) * a.Hq + hl[qb]) * a.Sq + i;
 				float* rp = a.o_part + row * D;
 #pragma unroll
 				for (int db = 0; db < DB; ++db)
@@ -627,7 +656,7 @@ hipError_t launch_fwd_split_t(bool bias, bool drop, KArgs& a, hipStream_t s) {
 	a.mtiles = (a.Sq + BM - 1) / BM;
 	int groups = a.B * a.Hkv;
 	a.xcd_remap = (groups % 8 == 0) ? 1 : 0;
-	dim3 grid((unsigned)(a.mtiles * a.B * a.Hq * a.nsplit)), block(NW * 64);
+	dim3 grid((unsigned)((a.pack_gqa ? a.B * a.Hkv : a.mtiles * a.B * a.Hq) * a.nsplit)), block(NW * 64);
 	if (bias && drop)
 		hipLaunchKernelGGL((fwd_kernel<T, D, NW, 1, 1, true, true, true>), grid, block, 0, s, a);
 	else if (bias)

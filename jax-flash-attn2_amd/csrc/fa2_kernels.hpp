@@ -35,6 +35,7 @@ struct KArgs {
 	int dq_makes_delta;  // the dQ kernel computes delta itself (and stores it for the dK/dV kernel)
 	// split forward (0 / 1 = off): key ranges of split_len keys, partial results in scratch
 	int nsplit, split_len;
+	int pack_gqa;     // split forward: one workgroup holds the rows of all q-heads of a kv-head
 	float* o_part;    // [nsplit, B, Hq, Sq, D] fp32
 	float* lse_part;  // [nsplit, B, Hq, Sq] fp32
 };

@@ -83,8 +83,13 @@ def test_bias_broadcast(bshape, D):
 		(1, 64, 2048, 2, 1, 256, torch.bfloat16, True, 2, 0.1),
 		(2, 5, 1024, 4, 2, 128, torch.bfloat16, False, 1, 0.0),
 		(1, 33, 777, 2, 2, 64, torch.bfloat16, True, None, 0.25),
+		# the rows of all q-heads of a kv-head share one workgroup when they fit one tile of 64 rows
+		(2, 7, 900, 8, 2, 128, torch.bfloat16, True, 8, 0.2),
+		(1, 16, 1024, 8, 2, 64, torch.float16, True, 2, 0.0),
+		(2, 3, 640, 12, 4, 256, torch.bfloat16, False, None, 0.0),
 	],
-	ids=["decode_gqa", "short_causal_fp16", "d256_bias_dropout", "bias_lds", "ragged_dropout"],
+	ids=["decode_gqa", "short_causal_fp16", "d256_bias_dropout", "bias_lds", "ragged_dropout", "packed_bias_dropout",
+	     "packed_kvhead_bias", "packed_d256"],
 )
 def test_short_query_split_over_keys(shape):
 	"""Sq <= 64 over many keys: the forward runs split over key ranges (partial results merged by
