@@ -60,25 +60,10 @@ FA2_DEV f32x16 mfma32(f16x8 a, f16x8 b, f32x16 c) {
 // The compiler does not know these statements are matrix products, so it adds
 // no wait states for them: the caller keeps a vector-ALU read of a result at
 // least two further matrix products away from the product that wrote it.
-//   mfma32_vz: C(VGPR) = A(VGPR) * B(AGPR)            first product of a chain
 //   mfma32_va: C(VGPR) += A(VGPR) * B(AGPR)
 //   mfma32_vc: C(VGPR) = A(VGPR) * B(AGPR) + C0(VGPR)   first product of a chain, from a start value
 //   mfma32_aa: C(AGPR) += A(VGPR) * B(VGPR)
 // BA: the B operand lives in an AGPR (else in a VGPR)
-template <bool BA>
-FA2_DEV void mfma32_vz(f32x16& c, bf16x8 a, bf16x8 b) {
-	if constexpr (BA)
-		asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
-	else
-		asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
-}
-template <bool BA>
-FA2_DEV void mfma32_vz(f32x16& c, f16x8 a, f16x8 b) {
-	if constexpr (BA)
-		asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
-	else
-		asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
-}
 template <bool BA>
 FA2_DEV void mfma32_va(f32x16& c, bf16x8 a, bf16x8 b) {
 	if constexpr (BA)
@@ -154,37 +139,15 @@ FA2_DEV int tile_off(int row, int chunk) {
 	return row * (D * 2) + ((chunk ^ swz<D>(row)) << 4);
 }
 
-// Fragment for the operand whose 32 rows/cols are tile rows and whose MFMA k
-// runs along D: lane l gets tile[row0 + l%32][16*ks + 8*(l/32) .. +7].
-template <typename T, int D>
-FA2_DEV typename T::V8 lds_frag(const FA2_LDS char* tile, int row0, int ks, int lane) {
-	int row = row0 + (lane & 31);
-	int chunk = 2 * ks + (lane >> 5);
-	return *(const FA2_LDS typename T::V8*)(tile + tile_off<D>(row, chunk));
-}
-
-// Transposed fragment: the operand's 32 rows/cols run along D (col0..col0+31)
-// and its MFMA k runs along tile rows.  k-slot (g = l/32, j) is tile row
-// row0 + 4g + j for j < 4 and row0 + 8 + 4g + (j-4) for j >= 4, which is the
-// order in which a 32x32 accumulator holds its rows - so an accumulator
-// packed to 16 bits is directly the other operand.
-// Built from two ds_read_b64_tr_b16: inside a block of 16 lanes, lane i
-// receives element i%4 of the 8-byte rows fetched by lanes 4j + i/4, j=0..3.
-template <typename T, int D>
-FA2_DEV typename T::V8 lds_frag_tr(const FA2_LDS char* tile, int row0, int col0, int lane) {
-	int i16 = lane & 15;
-	int g = lane >> 5;
-	int row = row0 + 4 * g + (i16 >> 2);
-	int col = col0 + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
-	typedef __attribute__((__vector_size__(4 * sizeof(short)))) short v4s;
-	const FA2_LDS char* p0 = tile + tile_off<D>(row, col >> 3) + ((col & 4) << 1);
-	const FA2_LDS char* p1 = tile + tile_off<D>(row + 8, col >> 3) + ((col & 4) << 1);
-	v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FA2_LDS v4s*)p0);
-	v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FA2_LDS v4s*)p1);
-	typedef __attribute__((__vector_size__(8 * sizeof(short)))) short v8s;
-	v8s both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-	return __builtin_bit_cast(typename T::V8, both);
-}
+// Fragments.  Operand whose 32 rows/cols are tile rows and whose MFMA k runs along D:
+// lane l holds tile[row0 + l%32][16*ks + 8*(l/32) .. +7], one 16-byte read at tile_off().
+// Transposed operand (its 32 rows/cols run along D, its MFMA k along tile rows):
+// k-slot (g = l/32, j) is tile row row0 + 4g + j for j < 4 and row0 + 8 + 4g + (j-4) for
+// j >= 4, which is the order in which a 32x32 accumulator holds its rows - so an
+// accumulator packed to 16 bits is directly the other operand.  It is built from two
+// ds_read_b64_tr_b16: inside a block of 16 lanes, lane i receives element i%4 of the
+// 8-byte rows fetched by lanes 4j + i/4, j = 0..3; the lane's own piece is rows
+// row0 + 4g + (l%16)/4 (+ 8), columns col0 + 16 ((l/16)%2) + 4 (l%4) .. +3.
 
 // Transposed fragment from two per-lane byte addresses (rows r and r + 8) plus a
 // compile-time byte offset.  Returned as raw bits; as_frag<T>() views them as the
@@ -232,51 +195,23 @@ FA2_DEV typename T::V8 as_frag(u32x4 x) {
 	return __builtin_bit_cast(typename T::V8, x);
 }
 
-// Copy a ROWS x D tile from global memory (row stride `stride` elements) into
-// a swizzled LDS tile without passing through registers.  Each wave-level
-// instruction moves 64 x 16 bytes; lane i lands at LDS slot base + i, so the
-// swizzle is applied by choosing which global chunk each lane fetches.  Rows
-// at or beyond `rows_valid` are fetched from the last valid row instead (the
-// caller masks their scores), so no lane reads out of bounds.
-// One wave-level 64 x 16-byte direct global->LDS copy: lane i fetches 16 bytes at
-// `src` and they land at LDS byte address `wave_dst` + 16 i (`wave_dst` is
-// wave-uniform).  Issued through inline assembly on purpose: the compiler then
-// does not model the copy as an LDS access in flight.  If it did, every wait for
-// an LDS read (s_waitcnt lgkmcnt) issued while a copy is outstanding would
-// drain ALL outstanding LDS reads instead of only those older than the one
-// needed, which defeats reading fragments several products ahead.  Completion
-// is awaited explicitly with wait_async_loads() before the workgroup barrier
-// that publishes the tile.
-FA2_DEV void lds_dma16(const char* src, FA2_LDS char* wave_dst) {
-	uint32_t m = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)wave_dst);
-	asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(m) : "memory", "m0");
-}
-
-template <int D, int ROWS, int NTHREADS>
-FA2_DEV void tile_load_async(FA2_LDS char* tile, const char* gbase, int64_t stride_bytes, int rows_valid, int tid) {
-	constexpr int CPR = D / 8;  // 16-byte chunks per row
-	constexpr int TOTAL = ROWS * CPR;
-	static_assert(TOTAL % NTHREADS == 0, "tile must divide over the workgroup");
-	int wave_base = (tid >> 6) << 6;
-	int lane = tid & 63;
-#pragma unroll
-	for (int it = 0; it < TOTAL / NTHREADS; ++it) {
-		int slot0 = it * NTHREADS + wave_base;  // wave-uniform
-		int slot = slot0 + lane;
-		int row = slot / CPR;
-		int pchunk = slot % CPR;
-		int chunk = pchunk ^ swz<D>(row);
-		int grow = row < rows_valid ? row : rows_valid - 1;
-		const char* src = gbase + (int64_t)grow * stride_bytes + (chunk << 4);
-		lds_dma16(src, tile + slot0 * 16);
-	}
-}
-
-// The same copy with the addressing hoisted out of the loop that streams tiles:
-// init() computes, once, this lane's byte offsets inside a full tile; load() then
-// issues one instruction per 64 x 16 bytes from a wave-uniform tile base (SGPR
-// pair) plus that 32-bit lane offset.  Ragged tiles (fewer than ROWS valid rows)
-// and strides too large for 32-bit offsets take the general path above.
+// Copy of a ROWS x D tile from global memory (row stride in bytes) into a swizzled LDS
+// tile without passing through registers.  Each wave-level instruction moves 64 x 16
+// bytes; lane i lands at LDS slot base + i, so the swizzle is applied by choosing which
+// global chunk each lane fetches.  Rows at or beyond the valid ones are fetched from the
+// last valid row instead (the caller masks their scores), so no lane reads out of bounds.
+// The copies are issued through inline assembly on purpose: the compiler then does not
+// model them as LDS accesses in flight.  If it did, every wait for an LDS read
+// (s_waitcnt lgkmcnt) issued while a copy is outstanding would drain ALL outstanding LDS
+// reads instead of only those older than the one needed, which defeats reading fragments
+// several products ahead.  Completion is awaited explicitly with wait_async_loads()
+// before the workgroup barrier that publishes the tile.
+// The addressing is hoisted out of the loop that streams tiles: init() computes, once,
+// this lane's byte offsets inside a tile; load() then issues one instruction per
+// 64 x 16 bytes from a wave-uniform tile base (SGPR pair) plus that 32-bit lane offset
+// (row stride x ROWS must fit 31 bits; the launcher checks).
+// One such instruction: lane i fetches 16 bytes at uniform_base + lane_off, they land at
+// LDS byte address wave_dst + 16 i (wave_dst is wave-uniform).
 FA2_DEV void lds_dma16_so(uint32_t lane_off, const char* uniform_base, FA2_LDS char* wave_dst) {
 	uint32_t m = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)wave_dst);
 	// s_nop 3: with s_mov that makes 5 wait states between a v_readfirstlane that produced the
@@ -377,10 +312,5 @@ FA2_DEV void philox4x32_rounds(uint32_t (&c)[4], uint32_t k0, uint32_t k1) {
 		c[3] = lo0;
 	}
 }
-
-struct Dropout {
-	uint32_t k0, k1, thr;
-	float inv_keep;  // 1 / (1 - p)
-};
 
 }  // namespace fa2
