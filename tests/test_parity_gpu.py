@@ -106,6 +106,46 @@ def test_short_query_split_over_keys(shape):
 	_run_case(B, Sq, Sk, Hq, Hkv, D, dtype, causal=causal, bias_shape=None if bh is None else (B, bh, Sq, Sk), p=p, seed=3)
 
 
+def _random_case(rng):
+	"""One configuration drawn from everything the operator accepts (sizes the fp64 oracle handles in well under a second)."""
+	r = int(rng.choice([1, 1, 2, 4]))
+	Hkv = int(rng.choice([1, 2, 3]))
+	Hq = Hkv * r
+	B = int(rng.choice([1, 2, 3]))
+	D = int(rng.choice([64, 64, 128, 128, 256, 40, 96]))
+	kind = rng.choice(["square", "square", "cross", "short_query", "one_tile"])
+	if kind == "square":
+		Sq = Sk = int(rng.integers(1, 400))
+	elif kind == "cross":
+		Sq, Sk = int(rng.integers(1, 300)), int(rng.integers(1, 600))
+	elif kind == "short_query":
+		Sq, Sk = int(rng.integers(1, 65)), int(rng.integers(512, 1400))
+	else:
+		Sq, Sk = int(rng.choice([64, 128, 256])), int(rng.choice([128, 256, 384]))
+	dtype = torch.bfloat16 if rng.random() < 0.6 else torch.float16
+	causal = bool(rng.random() < 0.5)
+	p = float(rng.choice([0.0, 0.0, 0.1, 0.3]))
+	bias_shape = bias_dtype = seqlens = None
+	extra = rng.choice(["none", "none", "bias", "bias", "seqlens"])
+	if extra == "bias":
+		bb = int(rng.choice([1, B]))
+		bh = int(rng.choice([1, Hq, Hkv]))
+		bias_shape = (bb, bh, Sq, Sk)
+		bias_dtype = torch.float32 if rng.random() < 0.25 else None
+	elif extra == "seqlens" and Sq == Sk:
+		seqlens = [int(rng.integers(0, Sk + 1)) for _ in range(B)]
+	return dict(B=B, Sq=Sq, Sk=Sk, Hq=Hq, Hkv=Hkv, D=D, dtype=dtype, causal=causal, bias_shape=bias_shape, p=p,
+	            seed=int(rng.integers(0, 2**31)), seqlens=seqlens, bias_dtype=bias_dtype, data_seed=int(rng.integers(0, 1000)))
+
+
+@pytest.mark.parametrize("chunk", range(6))
+def test_random_configurations(chunk):
+	"""Seeded sweep over shapes, head groupings, head dims, dtypes, causal, bias kinds, lengths and dropout."""
+	rng = np.random.default_rng(1000 + chunk)
+	for _ in range(8):
+		_run_case(**_random_case(rng))
+
+
 @pytest.mark.parametrize("D", [32, 80, 96, 160, 192])
 def test_other_head_dims(D):
 	"""Head dims between the built ones are zero-padded by the host layer (the reference pads
