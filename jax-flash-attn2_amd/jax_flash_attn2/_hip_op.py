@@ -203,6 +203,12 @@ class Plan:
 			self.dv = torch.empty_like(self.v, memory_format=torch.contiguous_format)
 			p.dout, p.dq, p.dk, p.dv = _t4(self.dout), _t4(self.dq), _t4(self.dk), _t4(self.dv)
 			need = self.lib.fa2_bwd_scratch_bytes(ctypes.byref(p))
+		else:
+			need = 0
+		# one buffer serves both calls: the backward needs its scratch, the forward uses scratch when it splits a
+		# short query over key ranges (the partial results do not outlive the forward call)
+		need = max(need, self.lib.fa2_fwd_scratch_bytes(ctypes.byref(p)))
+		if need:
 			self.scratch = torch.empty((max(need, 256),), dtype=torch.uint8, device=q.device)
 			p.scratch = self.scratch.data_ptr()
 			p.scratch_bytes = self.scratch.numel()
