@@ -95,9 +95,9 @@ void fill(const fa2_params* p, KArgs& a) {
 		                  ? 1
 		                  : 0;
 		// tiles of bias can be copied to LDS like K / V tiles: element type of q, 16-byte aligned
-		// rows, whole tiles of 64 keys, row stride within the 32-bit offsets of the tile copies
+		// rows of whole 16-byte pieces (8 keys), row stride within the 32-bit offsets of the tile copies
 		a.bias_lds = (p->bias_dtype == p->dtype && ((uintptr_t)p->bias % 16) == 0 && a.bias_sb % 16 == 0 && a.bias_sh % 16 == 0 &&
-		              a.bias_sm % 16 == 0 && a.bias_sm >= 0 && a.bias_sm <= 0x7fffffff / 256 && p->Sk % 64 == 0)
+		              a.bias_sm % 16 == 0 && a.bias_sm >= 0 && a.bias_sm <= 0x7fffffff / 256 && p->Sk % 8 == 0)
 		                 ? 1
 		                 : 0;
 	}

@@ -190,7 +190,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		if constexpr (BIAS_LDS) {
 			int hb = a.bias_group ? hk : hq;
 			const char* bb_ = a.bias + (int64_t)b * a.bias_sb + (int64_t)hb * a.bias_sh + (int64_t)m0 * a.bias_sm + (int64_t)n0 * 2;
-			bload.load(lds_bias + (step & 1) * BIAS_BYTES, bb_, a.bias_sm, rows, tid);
+			bload.load(lds_bias + (step & 1) * BIAS_BYTES, bb_, a.bias_sm, rows, tid, (a.Sk - n0) >> 3);
 		}
 	};
 	// per-row statistics of a tile: thread t < BMQ fetches lse, t in [BMQ, 2 BMQ) fetches delta
@@ -847,7 +847,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 		int row = w * (QB * 32) + c;
 		boff_lane = row * 128 + 8 * g;
 		bkey16 = swz<64>(row) << 4;
-		if (bias_lds && ntiles > 0) bload.load(lds + 4 * TILE_BYTES, bias_base + (int64_t)m0 * a.bias_sm, a.bias_sm, brows, tid);
+		if (bias_lds && ntiles > 0) bload.load(lds + 4 * TILE_BYTES, bias_base + (int64_t)m0 * a.bias_sm, a.bias_sm, brows, tid, a.Sk >> 3);
 	}
 
 	int koff[KS];
@@ -988,7 +988,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 				    if constexpr (BIAS_LDS) {
 					    if (bias_lds)
 						    bload.load(lds + 4 * TILE_BYTES + (buf ^ 1) * BIAS_BYTES, bias_base + (int64_t)m0 * a.bias_sm + (int64_t)n1 * 2,
-						               a.bias_sm, brows, tid);
+						               a.bias_sm, brows, tid, (a.Sk - n1) >> 3);
 				    }
 			    }
 		    },
@@ -1066,9 +1066,9 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 		a.mtiles = (a.Sk + C::KV_BN - 1) / C::KV_BN;
 		dim3 grid((unsigned)(a.mtiles * a.B * a.Hkv)), block(C::KV_NW * 64);
 		// typed variant: bias in the element type of q; where it stages the bias through LDS (D <= 128)
-		// it also needs 16-byte aligned rows and whole tiles of 128 keys
+		// it also needs 16-byte aligned rows of whole 16-byte pieces
 		bool typed = BIAS && a.bias_dtype == (std::is_same<T, BF16>::value ? 2 : 1);
-		if (D <= 128 && !(a.bias_lds && a.Sk % C::KV_BN == 0)) typed = false;
+		if (D <= 128 && !a.bias_lds) typed = false;
 		// with bias at D = 128 the streamed tiles are 64 rows, which leaves LDS room for the bias tiles
 		constexpr int QBV = (BIAS && D == 128) ? 2 : C::KV_QB;
 		if (typed)

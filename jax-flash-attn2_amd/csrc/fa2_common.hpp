@@ -229,23 +229,27 @@ struct TileLoader {
 	static_assert(TOTAL % NTHREADS == 0, "tile must divide over the workgroup");
 	uint32_t off[NIT];
 	int rows_state;  // the offsets clamp rows to [0, rows_state)
+	int cols_state;  // ... and 16-byte chunks of a row to [0, cols_state)
 
 	// stride_bytes * ROWS must fit 31 bits (the launcher checks)
-	FA2_DEV void init(int64_t stride_bytes, int tid, int rows_valid = ROWS) {
+	FA2_DEV void init(int64_t stride_bytes, int tid, int rows_valid = ROWS, int chunks_valid = CPR) {
 		rows_state = rows_valid;
+		cols_state = chunks_valid;
 #pragma unroll
 		for (int it = 0; it < NIT; ++it) {
 			int slot = it * NTHREADS + tid;
 			int row = slot / CPR;
 			int chunk = (slot % CPR) ^ swz<D>(row);
 			int grow = row < rows_valid ? row : rows_valid - 1;
-			off[it] = (uint32_t)grow * (uint32_t)stride_bytes + (uint32_t)(chunk << 4);
+			int gchunk = chunk < chunks_valid ? chunk : chunks_valid - 1;
+			off[it] = (uint32_t)grow * (uint32_t)stride_bytes + (uint32_t)(gchunk << 4);
 		}
 	}
-	// make the offsets fit a tile with rows_valid rows (wave-uniform; recomputes only on change)
-	FA2_DEV void fit(int64_t stride_bytes, int tid, int rows_valid) {
+	// make the offsets fit a tile with rows_valid rows of chunks_valid chunks (wave-uniform; recomputes only on change)
+	FA2_DEV void fit(int64_t stride_bytes, int tid, int rows_valid, int chunks_valid = CPR) {
 		rows_valid = rows_valid < ROWS ? rows_valid : ROWS;
-		if (rows_valid != rows_state) init(stride_bytes, tid, rows_valid);
+		chunks_valid = chunks_valid < CPR ? chunks_valid : CPR;
+		if (rows_valid != rows_state || chunks_valid != cols_state) init(stride_bytes, tid, rows_valid, chunks_valid);
 	}
 	// a wave-uniform pointer as an explicitly scalar value
 	static FA2_DEV const char* uniform(const char* p) {
@@ -258,9 +262,10 @@ struct TileLoader {
 		int wave_base = (tid >> 6) << 6;
 		lds_dma16_so(off[it], ub, tile + (it * NTHREADS + wave_base) * 16);
 	}
-	// whole tile; rows at or beyond rows_valid are fetched from the last valid row
-	FA2_DEV void load(FA2_LDS char* tile, const char* gbase, int64_t stride_bytes, int rows_valid, int tid) {
-		fit(stride_bytes, tid, rows_valid);
+	// whole tile; rows at or beyond rows_valid are fetched from the last valid row, 16-byte chunks at or
+	// beyond chunks_valid from the last valid chunk of their row
+	FA2_DEV void load(FA2_LDS char* tile, const char* gbase, int64_t stride_bytes, int rows_valid, int tid, int chunks_valid = CPR) {
+		fit(stride_bytes, tid, rows_valid, chunks_valid);
 		const char* ub = uniform(gbase);
 #pragma unroll
 		for (int it = 0; it < NIT; ++it) load_one(tile, ub, it, tid);

@@ -291,7 +291,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 		bkey16 = swz<64>(row) << 4;
 		if (bias_lds && ntiles > t_begin)
 			bload.load(lds + 4 * TILE_BYTES + (t_begin & 1) * BIAS_BYTES, bias_base + (int64_t)m0 * a.bias_sm + (int64_t)t_begin * BN * 2,
-			           a.bias_sm, brows, tid);
+			           a.bias_sm, brows, tid, (a.Sk - t_begin * BN) >> 3);
 	}
 
 	// Per-lane LDS byte offsets with the swizzle folded in, so that every fragment
@@ -531,7 +531,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 				    if constexpr (BIAS_LDS) {
 					    if (bias_lds)
 						    bload.load(lds + 4 * TILE_BYTES + (buf ^ 1) * BIAS_BYTES, bias_base + (int64_t)m0 * a.bias_sm + (int64_t)n1 * 2,
-						               a.bias_sm, brows, tid);
+						               a.bias_sm, brows, tid, (a.Sk - n1) >> 3);
 				    }
 			    }
 		    },
