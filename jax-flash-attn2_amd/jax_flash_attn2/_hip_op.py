@@ -100,6 +100,15 @@ def _prep_bias(bias):
 	return bias
 
 
+def _mask_to_bias(mask, q):
+	"""A 4-D boolean mask [B|1, H|1, Sq, Sk] as the additive bias where(mask, 0, finfo(dtype).min) - the recipe the
+	reference's documentation gives for general masks (README.md:188).  Its GPU path itself only takes the 2-D mask."""
+	m = mask.to(device=q.device)
+	m = m if m.dtype == torch.bool else m.ne(0)
+	zero = torch.zeros((), dtype=q.dtype, device=q.device)
+	return torch.where(m, zero, torch.full((), torch.finfo(q.dtype).min, dtype=q.dtype, device=q.device))
+
+
 def _seqlens_from_mask(attention_mask, q):
 	"""The reference's GPU path takes a right-padded 2-D validity mask [B, S] and
 	packs the valid tokens (_forward_triton.py:499-510).  Here the mask is reduced
@@ -259,6 +268,9 @@ def flash_attention(
 	compatibility; padded batches are always handled in-kernel from per-row
 	lengths, never by packing."""
 	del varlen_mode
+	if attention_mask is not None and attention_mask.dim() == 4:
+		assert bias is None, "Attention mask is not supported along with attention bias. Just use bias instead."
+		bias, attention_mask = _mask_to_bias(attention_mask, q), None
 	check_shapes(q, k, v, bias, attention_mask)
 	seqlens = _seqlens_from_mask(attention_mask, q)
 	return _FlashAttentionFn.apply(q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed)

@@ -147,7 +147,12 @@ def flash_attention(
 	varlen_mode: bool = True,
 ):
 	"""Same signature as the reference's `triton_flash_attention` (_flash_attention.py:125-157).
-	`dropout_seed` must be a Python int here: it becomes an attribute of the custom call."""
+	`dropout_seed` must be a Python int here: it becomes an attribute of the custom call.
+	A 4-D boolean mask becomes the bias where(mask, 0, finfo(dtype).min) (README.md:188)."""
+	if attention_mask is not None and attention_mask.ndim == 4:
+		assert bias is None, "Attention mask is not supported along with attention bias. Just use bias instead."
+		bias = jnp.where(attention_mask.astype(bool), jnp.zeros((), q.dtype), jnp.full((), jnp.finfo(q.dtype).min, q.dtype))
+		attention_mask = None
 	return flash_attention_call(q, k, v, attention_mask, bias, softmax_scale, dropout_prob, causal, dropout_seed, varlen_mode)
 
 

@@ -194,7 +194,9 @@ class FlashAttention:
 		if query.shape[1] != key.shape[1]:
 			if query.shape[1] == 1:
 				causal = False
-			attention_mask = None
+			# (the 2-D validity mask of the reference; a 4-D boolean mask is turned into a bias by the operator and kept)
+			if attention_mask is not None and len(attention_mask.shape) != 4:
+				attention_mask = None
 
 		if _is_jax_array(query):
 			from ._jax_op import flash_attention as op  # XLA-FFI custom calls into the same C ABI

@@ -172,6 +172,24 @@ def test_bias_dtypes_and_unaligned_rows():
 	_run_case(1, 96, 96, 2, 2, 256, torch.bfloat16, bias_shape=(1, 2, 96, 96))
 
 
+def test_boolean_4d_mask_through_the_facade():
+	"""A 4-D boolean mask is turned into the finfo.min bias of README.md:188 by the operator; also for Sq != Sk, where
+	the facade drops the reference's 2-D mask (flash_attention.py:239-242)."""
+	from jax_flash_attn2 import AttentionConfig, FlashAttention, Platform
+
+	attn = FlashAttention(AttentionConfig(platform=Platform.HIP))
+	for (Sq, Sk) in ((96, 96), (40, 200)):
+		q, k, v, do, _ = make_inputs(2, Sq, Sk, 4, 2, 64, torch.bfloat16, 12)
+		g = torch.Generator().manual_seed(5)
+		mask = torch.rand(2, 1, Sq, Sk, generator=g) < 0.7
+		mask[..., 0] = True  # every row keeps a key
+		bias = torch.where(mask, 0.0, float(torch.finfo(torch.bfloat16).min)).to(torch.bfloat16)
+		o_ref, _ = O.attention_fwd(f64(q), f64(k), f64(v), f64(bias))
+		out = attn(_dev(q), _dev(k), _dev(v), attention_mask=_dev(mask))
+		err = float(np.abs(out.float().cpu().numpy() - o_ref).max())
+		assert err <= TOL_O[torch.bfloat16], f"4-D mask Sq{Sq} Sk{Sk}: O max-abs {err:.3e}"
+
+
 def test_mask_as_finfo_min_bias():
 	"""Boolean mask -> where(mask, 0, finfo.min) bias (the README recipe) must equal key-length masking."""
 	B, S, H, D = 2, 192, 4, 64
