@@ -12,12 +12,12 @@
 // `make ffi XLA_FFI_INCLUDE=<dir>` and is not part of the default build.
 //
 // Operand convention (absent optional operands are passed as 0-element buffers):
-//   fa2_fwd_ffi : args q, k, v, bias, seqlens        rets o, lse
+//   fa2_fwd_ffi : args q, k, v, bias, seqlens        rets o, lse, scratch
 //   fa2_bwd_ffi : args q, k, v, bias, seqlens, o, lse, dout   rets dq, dk, dv, scratch
 //   attrs (both): scale f32, dropout_p f32, causal bool, seed i64, bias_group bool
 // All tensors are dense row-major as XLA lays them out: q/o/dout/dq [B,Sq,Hq,D],
 // k/v/dk/dv [B,Sk,Hkv,D], bias [B|1, H|1, Sq, Sk], lse [B,Hq,Sq] f32,
-// scratch [fa2_bwd_scratch_bytes] u8.
+// scratch u8: fa2_bwd_scratch_bytes for the backward, fa2_fwd_scratch_bytes (or any smaller size: no split) for the forward.
 #include <hip/hip_runtime.h>
 
 #include <cstring>
@@ -88,12 +88,16 @@ ffi::Error to_error(int rc) {
 }
 
 ffi::Error FwdImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::AnyBuffer v, ffi::AnyBuffer bias,
-                   ffi::AnyBuffer seqlens, ffi::Result<ffi::AnyBuffer> o, ffi::Result<ffi::AnyBuffer> lse, float scale,
-                   float dropout_p, bool causal, int64_t seed, bool bias_group) {
+                   ffi::AnyBuffer seqlens, ffi::Result<ffi::AnyBuffer> o, ffi::Result<ffi::AnyBuffer> lse,
+                   ffi::Result<ffi::AnyBuffer> scratch, float scale, float dropout_p, bool causal, int64_t seed,
+                   bool bias_group) {
 	fa2_params p;
 	if (auto e = fill_common(p, q, k, v, bias, seqlens, scale, dropout_p, causal, seed, bias_group); e.failure()) return e;
 	p.o = dense4(o->untyped_data(), q.dimensions());
 	p.lse = (float*)lse->untyped_data();
+	// optional: with fa2_fwd_scratch_bytes() of scratch a short query is split over key ranges
+	p.scratch = scratch->untyped_data();
+	p.scratch_bytes = scratch->size_bytes();
 	return to_error(fa2_fwd(&p, stream));
 }
 
@@ -142,6 +146,7 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(fa2_fwd_ffi, FwdImpl,
                                   .Arg<ffi::AnyBuffer>()  // seqlens
                                   .Ret<ffi::AnyBuffer>()  // o
                                   .Ret<ffi::AnyBuffer>()  // lse
+                                  .Ret<ffi::AnyBuffer>()  // scratch
                                   .Attr<float>("scale")
                                   .Attr<float>("dropout_p")
                                   .Attr<bool>("causal")

@@ -89,11 +89,28 @@ def _attrs(q, softmax_scale, dropout_prob, causal, dropout_seed, bias_group):
 	)
 
 
+def _fwd_scratch_bytes(q, k) -> int:
+	"""fa2_fwd_scratch_bytes for these shapes (host-only query; at least one aligned unit so the result is never empty)."""
+	import ctypes
+
+	from . import _lib
+
+	p = _lib.new_params()
+	p.B, p.Sq, p.Hq, p.D = (int(x) for x in q.shape)
+	p.Sk, p.Hkv = int(k.shape[1]), int(k.shape[2])
+	return max(int(_lib.load().fa2_fwd_scratch_bytes(ctypes.byref(p))), 256)
+
+
 def _fwd_call(q, k, v, bias, seqlens, attrs):
 	_register()
 	B, Sq, Hq, _ = q.shape
-	out_types = (jax.ShapeDtypeStruct(q.shape, q.dtype), jax.ShapeDtypeStruct((B, Hq, Sq), jnp.float32))
-	return _ffi.ffi_call("fa2_fwd_ffi", out_types)(q, k, v, bias, seqlens, **attrs)
+	out_types = (
+		jax.ShapeDtypeStruct(q.shape, q.dtype),
+		jax.ShapeDtypeStruct((B, Hq, Sq), jnp.float32),
+		jax.ShapeDtypeStruct((_fwd_scratch_bytes(q, k),), jnp.uint8),
+	)
+	out, lse, _ = _ffi.ffi_call("fa2_fwd_ffi", out_types)(q, k, v, bias, seqlens, **attrs)
+	return out, lse
 
 
 def _bwd_call(q, k, v, bias, seqlens, out, lse, dout, attrs):
