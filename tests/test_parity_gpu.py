@@ -363,3 +363,26 @@ def test_facade_forward_and_autograd():
 	with pytest.warns(UserWarning):
 		o4 = FlashAttention(AttentionConfig(platform=Platform.TRITON, backend=Backend.GPU))(qd.detach(), kd.detach(), vd.detach())
 	assert torch.equal(o4, attn(qd.detach(), kd.detach(), vd.detach()))
+
+
+def test_graph_capture_and_replay():
+	"""The library only enqueues kernels on the caller's stream (no allocation, no synchronisation), so a forward +
+	backward can be captured into a HIP graph; every replay must reproduce the eager results bit for bit."""
+	q, k, v, do, _ = make_inputs(2, 300, 300, 4, 2, 128, torch.bfloat16, 21)
+	plan = op.Plan(_dev(q), _dev(k), _dev(v), dout=_dev(do), causal=True, dropout_prob=0.1, dropout_seed=9)
+	plan.forward()
+	plan.backward()
+	torch.cuda.synchronize()
+	want = [t.clone() for t in (plan.out, plan.lse, plan.dq, plan.dk, plan.dv)]
+	graph = torch.cuda.CUDAGraph()
+	with torch.cuda.graph(graph):
+		plan.forward()
+		plan.backward()
+	for _ in range(3):
+		for t in (plan.out, plan.lse, plan.dq, plan.dk, plan.dv):
+			t.zero_()
+		torch.cuda.synchronize()
+		graph.replay()
+		torch.cuda.synchronize()
+		for got, ref in zip((plan.out, plan.lse, plan.dq, plan.dk, plan.dv), want):
+			assert torch.equal(got, ref)
