@@ -386,3 +386,40 @@ def test_graph_capture_and_replay():
 		torch.cuda.synchronize()
 		for got, ref in zip((plan.out, plan.lse, plan.dq, plan.dk, plan.dv), want):
 			assert torch.equal(got, ref)
+
+
+def test_concurrent_streams_and_threads():
+	"""No mutable global state: calls from several host threads on several streams give the results of running
+	them one after the other."""
+	import threading
+
+	cases = []
+	for n, (S, D, causal) in enumerate(((260, 64, True), (384, 128, False), (200, 128, True), (512, 64, False))):
+		q, k, v, do, _ = make_inputs(2, S, S, 4, 2, D, torch.bfloat16, 30 + n)
+		plan = op.Plan(_dev(q), _dev(k), _dev(v), dout=_dev(do), causal=causal)
+		plan.forward()
+		plan.backward()
+		torch.cuda.synchronize()
+		cases.append((plan, [t.clone() for t in (plan.out, plan.dq, plan.dk, plan.dv)]))
+	for plan, _ in cases:
+		for t in (plan.out, plan.dq, plan.dk, plan.dv):
+			t.zero_()
+	torch.cuda.synchronize()
+
+	def work(plan):
+		stream = torch.cuda.Stream()
+		with torch.cuda.stream(stream):
+			for _ in range(5):
+				plan.forward()
+				plan.backward()
+		stream.synchronize()
+
+	threads = [threading.Thread(target=work, args=(plan,)) for plan, _ in cases]
+	for t in threads:
+		t.start()
+	for t in threads:
+		t.join()
+	torch.cuda.synchronize()
+	for plan, want in cases:
+		for got, ref in zip((plan.out, plan.dq, plan.dk, plan.dv), want):
+			assert torch.equal(got, ref)
