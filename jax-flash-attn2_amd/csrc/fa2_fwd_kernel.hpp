@@ -652,7 +652,7 @@ struct FwdCfg {
 // Split forward: 2 waves x 32 rows per workgroup (the query is short), nsplit key ranges each.
 template <typename T, int D>
 hipError_t launch_fwd_split_t(bool bias, bool drop, KArgs& a, hipStream_t s) {
-	constexpr int NW = 2, BM = NW * 32;
+	constexpr int NW = D == 256 ? 4 : 2, BM = NW * 32;  // (D = 256: four waves, the tile copies need the threads)
 	a.mtiles = (a.Sq + BM - 1) / BM;
 	int groups = a.B * a.Hkv;
 	a.xcd_remap = (groups % 8 == 0) ? 1 : 0;
