@@ -688,7 +688,8 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 // ---------------------------------------------------------------------------
 // dQ
 // ---------------------------------------------------------------------------
-template <typename T, int D, int NW, int QB, int WPS, bool BIAS, bool DROP>
+// BLDS: the bias goes through LDS as in the forward kernel (conditions checked by the launcher)
+template <typename T, int D, int NW, int QB, int WPS, bool BIAS, bool DROP, bool BLDS = false>
 __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 	typedef typename T::V8 V8;
 	constexpr int BM = NW * QB * 32;
@@ -700,7 +701,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 	constexpr int TILE_BYTES = BN * D * 2;
 
 	// bias tiles through LDS as in the forward kernel
-	constexpr bool BIAS_LDS = BIAS && D <= 128;
+	constexpr bool BIAS_LDS = BIAS && BLDS && D <= 128;
 	constexpr int BIAS_BYTES = BIAS_LDS ? BM * BN * 2 : 0;
 	static_assert(BN == 64, "bias tiles use the 64-element row geometry");
 	__shared__ __attribute__((aligned(1024))) char smem[4 * TILE_BYTES + 2 * BIAS_BYTES];
@@ -838,7 +839,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 		int hb = a.bias_group ? hk : h;
 		bias_base = a.bias + (int64_t)b * a.bias_sb + (int64_t)hb * a.bias_sh;
 	}
-	const bool bias_lds = BIAS_LDS && a.bias_lds;
+	constexpr bool bias_lds = BIAS_LDS;
 	TileLoader<64, BM, NT> bload;
 	int brows = 0, boff_lane = 0, bkey16 = 0;
 	if constexpr (BIAS_LDS) {
@@ -870,14 +871,13 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 		constexpr bool MASKED = decltype(masked_tag)::value;
 #pragma unroll
 		for (int kb = 0; kb < KB; ++kb) {
-			f32x4 bv[BIAS ? QB : 1][4];
-			if (BIAS_LDS && bias_lds) {
+			f32x4 bv[BIAS && !BIAS_LDS ? QB : 1][4];
+			typename T::V4 bvl[BIAS_LDS ? 4 : 1];  // from LDS, kept in the element type until used (half the registers)
+			if constexpr (BIAS_LDS) {
 				static_assert(!BIAS_LDS || QB == 1, "");
 #pragma unroll
-				for (int aa = 0; aa < 4; ++aa) {
-					typename T::V4 x = *(const FA2_LDS typename T::V4*)(bt + boff_lane + (((kb * 4 + aa) << 4) ^ bkey16));
-					bv[0][aa] = __builtin_convertvector(x, f32x4);
-				}
+				for (int aa = 0; aa < 4; ++aa)
+					bvl[aa] = *(const FA2_LDS typename T::V4*)(bt + boff_lane + (((kb * 4 + aa) << 4) ^ bkey16));
 			} else if constexpr (BIAS) {
 #pragma unroll
 				for (int qb = 0; qb < QB; ++qb) {
@@ -940,7 +940,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 						int i = 4 * aa + e;
 						float p;
 						if constexpr (BIAS)
-							p = exp2_fast((__builtin_fmaf(s[qb][i], c1, bv[qb][aa][e]) - lse_r[qb]) * kLog2e);
+							p = exp2_fast((__builtin_fmaf(s[qb][i], c1, BIAS_LDS ? (float)bvl[aa][e] : bv[qb][aa][e]) - lse_r[qb]) * kLog2e);
 						else
 							p = exp2_fast(__builtin_fmaf(s[qb][i], c1, -lse_r[qb]));
 						if constexpr (MASKED) {
@@ -1059,7 +1059,10 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 	auto launch_dq = [&]() {
 		a.mtiles = (a.Sq + C::DQ_BM - 1) / C::DQ_BM;
 		dim3 grid((unsigned)(a.mtiles * a.B * a.Hq)), block(C::DQ_NW * 64);
-		hipLaunchKernelGGL((bwd_dq_kernel<T, D, C::DQ_NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP>), grid, block, 0, s, a);
+		if (BIAS && a.bias_lds && D <= 128)
+			hipLaunchKernelGGL((bwd_dq_kernel<T, D, C::DQ_NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, BIAS>), grid, block, 0, s, a);
+		else
+			hipLaunchKernelGGL((bwd_dq_kernel<T, D, C::DQ_NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, false>), grid, block, 0, s, a);
 	};
 	if (fused_delta) launch_dq();
 	if (a.stages & 2) {

@@ -96,7 +96,9 @@ FA2_DEV f32x4 load_bias4(const char* rowp, int col, int dtype, bool vec_ok, int 
 // fp32 and its logsumexp) in scratch for fwd_combine_kernel.  For few query rows and many
 // keys (decoding, short cross-attention queries), where one workgroup per row tile would
 // leave most of the chip idle.
-template <typename T, int D, int NW, int QB, int WPS, bool BIAS, bool DROP, bool SPLIT = false>
+// BLDS: the bias goes through LDS (the launcher has checked element type, alignment and the key
+// count); otherwise every lane loads its bias values from global memory.
+template <typename T, int D, int NW, int QB, int WPS, bool BIAS, bool DROP, bool SPLIT = false, bool BLDS = false>
 __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 	typedef typename T::V8 V8;
 	constexpr int BM = NW * QB * 32;
@@ -109,7 +111,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 
 	// Bias tiles (BM rows x 64 keys, element type of q) go through LDS as well when there is
 	// room: read from global memory one row per lane, a wave's load touches 32 cache lines.
-	constexpr bool BIAS_LDS = BIAS && D <= 128;
+	constexpr bool BIAS_LDS = BIAS && BLDS && D <= 128;
 	constexpr int BIAS_BYTES = BIAS_LDS ? BM * BN * 2 : 0;
 	static_assert(BN == 64, "bias tiles use the 64-element row geometry");
 	__shared__ __attribute__((aligned(1024))) char smem[4 * TILE_BYTES + 2 * BIAS_BYTES];
@@ -279,7 +281,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 		int hb = a.bias_group ? hk : h;
 		bias_base = a.bias + (int64_t)b * a.bias_sb + (int64_t)hb * a.bias_sh;
 	}
-	const bool bias_lds = BIAS_LDS && a.bias_lds && !pack;
+	constexpr bool bias_lds = BIAS_LDS;
 	TileLoader<64, BM, NT> bload;
 	int brows = 0, boff_lane = 0, bkey16 = 0;
 	if constexpr (BIAS_LDS) {
@@ -657,7 +659,12 @@ hipError_t launch_fwd_split_t(bool bias, bool drop, KArgs& a, hipStream_t s) {
 	int groups = a.B * a.Hkv;
 	a.xcd_remap = (groups % 8 == 0) ? 1 : 0;
 	dim3 grid((unsigned)((a.pack_gqa ? a.B * a.Hkv : a.mtiles * a.B * a.Hq) * a.nsplit)), block(NW * 64);
-	if (bias && drop)
+	const bool blds = bias && a.bias_lds && D <= 128 && !a.pack_gqa;
+	if (blds && drop)
+		hipLaunchKernelGGL((fwd_kernel<T, D, NW, 1, 1, true, true, true, true>), grid, block, 0, s, a);
+	else if (blds)
+		hipLaunchKernelGGL((fwd_kernel<T, D, NW, 1, 1, true, false, true, true>), grid, block, 0, s, a);
+	else if (bias && drop)
 		hipLaunchKernelGGL((fwd_kernel<T, D, NW, 1, 1, true, true, true>), grid, block, 0, s, a);
 	else if (bias)
 		hipLaunchKernelGGL((fwd_kernel<T, D, NW, 1, 1, true, false, true>), grid, block, 0, s, a);
@@ -680,7 +687,12 @@ hipError_t launch_fwd_t(bool bias, bool drop, KArgs& a, hipStream_t s) {
 	a.xcd_remap = (groups % 8 == 0) ? 1 : 0;
 	if (bias && a.bias_sh == 0 && a.B % 8 == 0) a.xcd_remap = 2;
 	dim3 grid((unsigned)(a.mtiles * a.B * a.Hq)), block(C::NW * 64);
-	if (bias && drop)
+	const bool blds = bias && a.bias_lds && D <= 128;
+	if (blds && drop)
+		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, C::WPS, true, true, false, true>), grid, block, 0, s, a);
+	else if (blds)
+		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, C::WPS, true, false, false, true>), grid, block, 0, s, a);
+	else if (bias && drop)
 		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, C::WPS, true, true>), grid, block, 0, s, a);
 	else if (bias)
 		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, C::WPS, true, false>), grid, block, 0, s, a);
