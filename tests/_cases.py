@@ -48,7 +48,8 @@ def check_grads(got, ref, what=""):
 		if np.abs(b).max() <= 1e-10:
 			# a gradient that is zero up to fp64 rounding (e.g. a single key: dS = P (dP - delta) = 0) may come
 			# back as rounding noise of delta
-			assert np.abs(a).max() <= 1e-3, f"{what}: {name} should be zero"
+			# (delta is formed from O rounded to 16 bits: up to 2^-8 of |dP| survives the subtraction)
+			assert np.abs(a).max() <= 1e-2, f"{what}: {name} should be zero"
 			continue
 		e = O.rel_l2(a, b)
 		assert e <= TOL_GRAD_REL_L2, f"{what}: {name} rel-L2 {e:.3e} > {TOL_GRAD_REL_L2}"
