@@ -170,7 +170,19 @@ def flash_attention(
 		assert bias is None, "Attention mask is not supported along with attention bias. Just use bias instead."
 		bias = jnp.where(attention_mask.astype(bool), jnp.zeros((), q.dtype), jnp.full((), jnp.finfo(q.dtype).min, q.dtype))
 		attention_mask = None
-	return flash_attention_call(q, k, v, attention_mask, bias, softmax_scale, dropout_prob, causal, dropout_seed, varlen_mode)
+	# head dims other than 64 / 128 / 256: zero-pad to the next one (the reference pads to the next power of two,
+	# _forward_triton.py:525-526); pad and slice are differentiated by jax, the scale keeps the true head dim
+	D0 = q.shape[-1]
+	D = next((d for d in (64, 128, 256) if D0 <= d), None)
+	if D is None:
+		raise ValueError(f"head dim {D0} is not supported (at most 256)")
+	if D != D0:
+		if softmax_scale is None:
+			softmax_scale = 1.0 / math.sqrt(D0)
+		pad = ((0, 0), (0, 0), (0, 0), (0, D - D0))
+		q, k, v = jnp.pad(q, pad), jnp.pad(k, pad), jnp.pad(v, pad)
+	out = flash_attention_call(q, k, v, attention_mask, bias, softmax_scale, dropout_prob, causal, dropout_seed, varlen_mode)
+	return out if D == D0 else out[..., :D0]
 
 
 def dropout_mask(B, H, Sq, Sk, dropout_prob, dropout_seed):
