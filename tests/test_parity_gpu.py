@@ -172,6 +172,28 @@ def test_bias_dtypes_and_unaligned_rows():
 	_run_case(1, 96, 96, 2, 2, 256, torch.bfloat16, bias_shape=(1, 2, 96, 96))
 
 
+def test_rows_masked_entirely_by_finfo_min_bias_stay_finite():
+	"""A query row whose keys are all masked through the finfo.min bias (a padded query under the README mask
+	recipe) gives the plain average of V - every score is the same huge negative number - and finite gradients;
+	the valid rows are unaffected."""
+	dtype = torch.bfloat16
+	B, S, H, D = 2, 192, 2, 64
+	q, k, v, do, _ = make_inputs(B, S, S, H, H, D, dtype, 17)
+	fill = float(torch.finfo(dtype).min)
+	bias = torch.zeros(B, 1, S, S)
+	bias[:, :, 150:, :] = fill          # rows 150.. see nothing
+	bias[:, :, :, 170:] = fill          # keys 170.. are padding
+	bias = bias.to(dtype)
+	o, lse = op.fwd(_dev(q), _dev(k), _dev(v), _dev(bias))
+	g = op.bwd(_dev(q), _dev(k), _dev(v), o, lse, _dev(do), _dev(bias))
+	torch.cuda.synchronize()
+	assert torch.isfinite(o).all() and all(torch.isfinite(x).all() for x in g)
+	want = v.float().mean(dim=1, keepdim=True).expand(B, S - 150, H, D)
+	assert float((o[:, 150:].float().cpu() - want).abs().max()) <= TOL_O[dtype]
+	o_ref, lse_ref = O.attention_fwd(f64(q[:, :150]), f64(k), f64(v), f64(bias[:, :, :150]))
+	assert float(np.abs(o[:, :150].float().cpu().numpy() - o_ref).max()) <= TOL_O[dtype]
+
+
 def test_boolean_4d_mask_through_the_facade():
 	"""A 4-D boolean mask is turned into the finfo.min bias of README.md:188 by the operator; also for Sq != Sk, where
 	the facade drops the reference's 2-D mask (flash_attention.py:239-242)."""
