@@ -48,7 +48,9 @@ enum {
 	                             (_forward_triton.py:474-481)                    */
 	FA2_EUNSUPPORTED = -10,   /* head dim not in {64, 128, 256}                  */
 	FA2_ESCRATCH = -11,       /* backward scratch missing or too small           */
-	FA2_EHIP = -12            /* HIP runtime reported a launch error             */
+	FA2_EHIP = -12,           /* HIP runtime reported a launch error             */
+	FA2_ESCRATCH_STATIC = -13 /* fa2_bwd_static: the call needs more than
+	                             FA2_STATIC_SCRATCH_BYTES of scratch             */
 };
 
 typedef struct fa2_tensor {
@@ -130,6 +132,20 @@ int fa2_bwd_stages(const fa2_params* p, void* hip_stream, int stages);
 
 /* Bytes of scratch fa2_bwd needs for these dimensions (0 on invalid params). */
 size_t fa2_bwd_scratch_bytes(const fa2_params* p);
+
+/* fa2_bwd for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  p->scratch / p->scratch_bytes are ignored: the
+ * scratch (delta, [B, Hq, Sq] fp32) lives in a buffer of FA2_STATIC_SCRATCH_BYTES
+ * built into the library, one copy per GPU, held until the process ends.  Calls
+ * whose fa2_bwd_scratch_bytes() exceeds that limit (B * Hq * Sq > 4 Mi rows) fail
+ * with FA2_ESCRATCH_STATIC and launch nothing.  The call itself allocates and
+ * frees nothing and launches the same two kernels as fa2_bwd.  All calls on one
+ * GPU share the buffer: two calls that overlap in time on the same GPU (different
+ * streams or threads) race on it - order them.  The first call on each GPU looks
+ * up the buffer's device address; make that call outside graph capture. */
+#define FA2_STATIC_SCRATCH_BYTES (16u << 20)
+int fa2_bwd_static(const fa2_params* p, void* hip_stream);
 
 /* keep[b,h,i,j] (uint8, contiguous [B,Hq,Sq,Sk]) of the dropout mask the
  * kernels apply for (seed, p_drop); for validation against the Philox

@@ -5,7 +5,13 @@
 #include <math.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "fa2_kernels.hpp"
+
+// Scratch of fa2_bwd_static(): one copy per GPU the library runs on, held until the process
+// ends.  In host code this name is only a handle for hipGetSymbolAddress(), never an address.
+static __device__ __align__(256) unsigned char scratch[FA2_STATIC_SCRATCH_BYTES];
 
 namespace {
 
@@ -35,7 +41,8 @@ KTensor conv(const fa2_tensor& t) {
 	return k;
 }
 
-int validate(const fa2_params* p, int which) {
+// own_scratch: the backward brings its scratch itself (fa2_bwd_static), p->scratch is not looked at
+int validate(const fa2_params* p, int which, bool own_scratch = false) {
 	if (!p || p->struct_size < sizeof(fa2_params)) return FA2_EINVAL_STRUCT;
 	if (p->dtype != FA2_FP16 && p->dtype != FA2_BF16) return FA2_EINVAL_DTYPE;
 	if (p->B <= 0 || p->Sq <= 0 || p->Sk <= 0 || p->Hq <= 0 || p->Hkv <= 0 || p->D <= 0) return FA2_EINVAL_SHAPE;
@@ -64,7 +71,11 @@ int validate(const fa2_params* p, int which) {
 		if ((rc = check_tensor(p->dk, true))) return rc;
 		if ((rc = check_tensor(p->dv, true))) return rc;
 		size_t need = fa2_bwd_scratch_bytes(p);
-		if (!p->scratch || ((uintptr_t)p->scratch & 255) || p->scratch_bytes < need) return FA2_ESCRATCH;
+		if (own_scratch) {
+			if (need > FA2_STATIC_SCRATCH_BYTES) return FA2_ESCRATCH_STATIC;
+		} else if (!p->scratch || ((uintptr_t)p->scratch & 255) || p->scratch_bytes < need) {
+			return FA2_ESCRATCH;
+		}
 	}
 	return FA2_OK;
 }
@@ -207,9 +218,7 @@ int fa2_fwd(const fa2_params* p, void* hip_stream) {
 
 int fa2_bwd(const fa2_params* p, void* hip_stream) { return fa2_bwd_stages(p, hip_stream, 7); }
 
-int fa2_bwd_stages(const fa2_params* p, void* hip_stream, int stages) {
-	int rc = validate(p, 1);
-	if (rc) return rc;
+static int bwd_launch(const fa2_params* p, void* hip_stream, int stages, void* scratch_ptr) {
 	KArgs a;
 	fill(p, a);
 	a.stages = stages & 7;
@@ -217,9 +226,41 @@ int fa2_bwd_stages(const fa2_params* p, void* hip_stream, int stages) {
 	a.dq = conv(p->dq);
 	a.dk = conv(p->dk);
 	a.dv = conv(p->dv);
-	a.delta = (float*)p->scratch;
+	a.delta = (float*)scratch_ptr;
 	hipError_t e = fa2::launch_bwd(p->dtype, p->D, p->bias != nullptr, p->p_drop > 0.f, a, (hipStream_t)hip_stream);
 	return e == hipSuccess ? FA2_OK : FA2_EHIP;
+}
+
+int fa2_bwd_stages(const fa2_params* p, void* hip_stream, int stages) {
+	int rc = validate(p, 1);
+	if (rc) return rc;
+	return bwd_launch(p, hip_stream, stages, p->scratch);
+}
+
+// Device address of `scratch` on the current device, looked up once per device.
+static int static_scratch_ptr(void** out) {
+	constexpr int kMaxDevices = 64;
+	static void* ptrs[kMaxDevices];
+	static std::mutex mu;
+	int dev = -1;
+	if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return FA2_EHIP;
+	std::lock_guard<std::mutex> lock(mu);
+	if (!ptrs[dev]) {
+		void* ptr = nullptr;
+		if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return FA2_EHIP;
+		ptrs[dev] = ptr;
+	}
+	*out = ptrs[dev];
+	return FA2_OK;
+}
+
+int fa2_bwd_static(const fa2_params* p, void* hip_stream) {
+	int rc = validate(p, 1, /*own_scratch=*/true);
+	if (rc) return rc;
+	void* ptr = nullptr;
+	if ((rc = static_scratch_ptr(&ptr))) return rc;
+	// delta is written in full by the first kernel before the second reads it: nothing to clear
+	return bwd_launch(p, hip_stream, 7, ptr);
 }
 
 int fa2_dropout_mask(const fa2_params* p, uint8_t* keep, void* hip_stream) {
@@ -247,6 +288,7 @@ const char* fa2_strerror(int code) {
 		case FA2_EUNSUPPORTED: return "head dim must be 64, 128 or 256";
 		case FA2_ESCRATCH: return "backward scratch buffer missing, misaligned or too small";
 		case FA2_EHIP: return "HIP launch failed";
+		case FA2_ESCRATCH_STATIC: return "fa2_bwd_static: B * Hq * Sq * 4 bytes exceed the 16 MiB built-in scratch";
 		default: return "unknown error";
 	}
 }

@@ -64,6 +64,7 @@ EXPORTS = (
 	"fa2_fwd",
 	"fa2_bwd",
 	"fa2_bwd_stages",
+	"fa2_bwd_static",
 	"fa2_bwd_scratch_bytes",
 	"fa2_fwd_scratch_bytes",
 	"fa2_dropout_mask",
@@ -103,6 +104,8 @@ def load() -> ctypes.CDLL:
 		lib.fa2_bwd.restype = ctypes.c_int
 		lib.fa2_bwd_stages.argtypes = [pp, ctypes.c_void_p, ctypes.c_int]
 		lib.fa2_bwd_stages.restype = ctypes.c_int
+		lib.fa2_bwd_static.argtypes = [pp, ctypes.c_void_p]
+		lib.fa2_bwd_static.restype = ctypes.c_int
 		lib.fa2_bwd_scratch_bytes.argtypes = [pp]
 		lib.fa2_bwd_scratch_bytes.restype = ctypes.c_size_t
 		lib.fa2_fwd_scratch_bytes.argtypes = [pp]
