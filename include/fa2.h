@@ -66,12 +66,8 @@ typedef struct fa2_params {
 	int32_t B, Sq, Sk, Hq, Hkv, D;
 	int32_t causal;         /* bottom-right aligned: j <= i + Sk - Sq
 	                           (_forward_triton.py:127-132)                */
-	float scale;            /* softmax scale, applied to q.k^T; must be > 0.  Without bias the forward kernel keeps
-	                           scale*log2(e)*q and the dK/dV kernel scale*log2(e)*k in the element type (for fp16 these
-	                           products must stay below 65504): every term of a score then carries one more rounding
-	                           of 2^-9 (bf16) / 2^-12 (fp16) relative - the error level of an attention that rounds
-	                           the scores to the element type.  Measured against fp64 on bf16 inputs: |lse error| 4e-3
-	                           for scores within +-7, 3e-2 within +-20, 1.3e-1 within +-80 (1e-5 without that step) */
+	float scale;            /* softmax scale, must be > 0; applied to the fp32 result of q.k^T,
+	                           as the reference does (_forward_triton.py:281)  */
 	float p_drop;           /* dropout probability in [0,1)                */
 	uint64_t seed;          /* Philox key for the dropout keep-mask        */
 

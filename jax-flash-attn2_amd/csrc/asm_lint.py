@@ -1,0 +1,150 @@
+#!/usr/bin/env python3
+"""Build-time check of the register hazards around matrix products issued as inline assembly.
+
+The kernels issue some v_mfma instructions through inline assembly (so that the register file
+of every operand can be pinned).  The compiler treats such a statement as opaque: it neither
+pads the wait states a matrix product needs nor keeps its source registers untouched while
+the product runs.  The sources keep those distances by construction; this script reads the
+assembly text the compiler emits for the same translation unit (`hipcc -S`, no binary is
+taken apart) and fails the build when a later compiler version, or an edit, breaks one.
+
+Rules, per kernel, in program-text order (a v_mfma between `;;#ASMSTART` and `;;#ASMEND`):
+  R1  the product's C operand, when it is not also its destination, is not written by any
+      instruction before one further v_mfma has been issued (or 7 wait states have passed):
+      an 8-pass product reads C while it runs, and the hardware does not hold back a
+      vector-ALU write to those registers;
+  R2  the product's destination is not read by anything but a v_mfma C operand before two
+      further v_mfma have been issued (or 11 wait states have passed).
+A wait state is one instruction; `s_nop N` counts N + 1.
+
+Usage: asm_lint.py FILE.s [FILE.s ...]   (exit status 1 and one line per violation)
+"""
+
+from __future__ import annotations
+
+import re
+import sys
+
+R1_WAIT = 7
+R2_WAIT = 11
+
+_LABEL = re.compile(r"^([A-Za-z_][\w$]*):\s*(;.*)?$")  # a function label (local labels start with a dot)
+_REG = re.compile(r"\b([va])(?:\[(\d+):(\d+)\]|(\d+))")
+
+
+def _regs(operand: str):
+	"""Set of (file, index) named by one operand."""
+	out = set()
+	for m in _REG.finditer(operand):
+		f = m.group(1)
+		if m.group(4) is not None:
+			out.add((f, int(m.group(4))))
+		else:
+			out.update((f, i) for i in range(int(m.group(2)), int(m.group(3)) + 1))
+	return out
+
+
+def _split(line: str):
+	line = line.split(";")[0].strip()
+	if not line or line.endswith(":") or line.startswith("."):
+		return None, []
+	parts = line.split(None, 1)
+	ops = [o.strip() for o in parts[1].split(",")] if len(parts) > 1 else []
+	return parts[0], ops
+
+
+def _writes(mn: str, ops):
+	"""Registers an instruction writes (vector files only)."""
+	if not ops:
+		return set()
+	if mn.startswith(("v_cmp", "v_readfirstlane", "v_readlane", "s_", "ds_write", "ds_store", "global_store", "buffer_store",
+	                  "flat_store", "global_atomic", "global_load_lds", "buffer_wbl2", "buffer_inv")):
+		return set()
+	if mn.startswith(("v_swap", "v_permlane")):
+		return _regs(ops[0]) | (_regs(ops[1]) if len(ops) > 1 else set())
+	if mn.startswith(("v_", "ds_read", "ds_load", "global_load", "buffer_load", "flat_load", "scratch_load")):
+		return _regs(ops[0])
+	return set()
+
+
+def _reads(mn: str, ops):
+	if not ops:
+		return set()
+	if mn.startswith(("ds_write", "ds_store", "global_store", "buffer_store", "flat_store", "global_atomic", "global_load_lds")):
+		src = ops
+	else:
+		src = ops[1:]
+	out = set()
+	for o in src:
+		out |= _regs(o)
+	return out
+
+
+def lint(path: str):
+	problems = []
+	kernel = "?"
+	in_asm = False
+	pending = []  # dicts: line, c (set or None), dst (set), mfma_since, wait_since
+	with open(path) as f:
+		for ln, raw in enumerate(f, 1):
+			s = raw.strip()
+			if s.startswith(";;#ASMSTART"):
+				in_asm = True
+				continue
+			if s.startswith(";;#ASMEND"):
+				in_asm = False
+				continue
+			m = _LABEL.match(s)
+			if m:
+				kernel = m.group(1)
+				pending = []
+				continue
+			mn, ops = _split(raw)
+			if mn is None:
+				continue
+			is_mfma = mn.startswith("v_mfma")
+			w, r = _writes(mn, ops), _reads(mn, ops)
+			if is_mfma and len(ops) >= 4:
+				r_nonc = _regs(ops[1]) | _regs(ops[2])
+			else:
+				r_nonc = r
+			for p in pending:
+				if p["c"] and p["mfma"] < 1 and p["wait"] < R1_WAIT and (w & p["c"]):
+					problems.append(f"{path}:{ln}: {kernel}: R1: `{s}` writes the C operand of the product at line {p['line']}")
+				if p["mfma"] < 2 and p["wait"] < R2_WAIT and (r_nonc & p["dst"]):
+					problems.append(f"{path}:{ln}: {kernel}: R2: `{s}` reads the result of the product at line {p['line']}")
+			# advance the clocks
+			step = 1
+			if mn == "s_nop" and ops:
+				try:
+					step = int(ops[0], 0) + 1
+				except ValueError:
+					pass
+			for p in pending:
+				p["wait"] += step
+				if is_mfma:
+					p["mfma"] += 1
+			pending = [p for p in pending if p["mfma"] < 2 and p["wait"] < max(R1_WAIT, R2_WAIT)]
+			if is_mfma and in_asm and len(ops) >= 4:
+				dst, c = _regs(ops[0]), _regs(ops[3])
+				pending.append({"line": ln, "c": (c if c and c != dst else None), "dst": dst, "mfma": 0, "wait": 0})
+	return problems
+
+
+def main(argv):
+	if len(argv) < 2:
+		print(__doc__)
+		return 2
+	bad = []
+	for path in argv[1:]:
+		bad += lint(path)
+	for b in bad:
+		print(b)
+	if bad:
+		print(f"asm_lint: {len(bad)} hazard(s)")
+		return 1
+	return 0
+
+
+if __name__ == "__main__":
+	sys.exit(main(sys.argv))

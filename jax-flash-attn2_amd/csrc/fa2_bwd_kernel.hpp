@@ -71,9 +71,10 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	// S / dP accumulators in VGPRs) when the AGPR file holds the former; the bias and dropout
 	// variants need the registers for other things and leave the choice to the compiler.
 	constexpr bool KV_AGPR = 2 * KS * 4 + 2 * DB * 16 <= 256 && !BIAS && !DROP;
-	// On that path the elementwise stage is shortened: K is pre-multiplied by scale * log2(e)
-	// and the chains of S and dP start from -lse and -delta instead of 0, so that
-	// P = exp2(S accumulator) and dS = P * (dP accumulator) need no further arithmetic.
+	// On that path the elementwise stage is shortened: the chains of S and dP start from
+	// -lse / (scale log2(e)) and -delta instead of 0, so that P = exp2(c1 * S accumulator) and
+	// dS = P * (dP accumulator).  The factor c1 = scale * log2(e) is applied to the fp32
+	// accumulator, as the reference scales the fp32 result of its dot (_backward_triton.py:554-559).
 	constexpr bool FOLD = KV_AGPR;
 
 	// A bias in the element type of q is streamed through LDS as tiles of BMQ rows x BN keys
@@ -144,16 +145,6 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		}
 	}
 
-	if constexpr (FOLD) {
-		const float kc = a.scale * kLog2e;
-#pragma unroll
-		for (int ks = 0; ks < KS; ++ks) {
-			typename T::V8 x = kf[ks];
-			kf[ks] = pack8<T>((float)x[0] * kc, (float)x[1] * kc, (float)x[2] * kc, (float)x[3] * kc, (float)x[4] * kc,
-			                  (float)x[5] * kc, (float)x[6] * kc, (float)x[7] * kc);
-		}
-	}
-
 	f32x16 dk[DB], dv[DB];
 #pragma unroll
 	for (int db = 0; db < DB; ++db)
@@ -172,6 +163,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	const int steps = nq * r;
 
 	const float c1 = BIAS ? a.scale : a.scale * kLog2e;
+	const float inv_scale = 1.f / a.scale;
 
 	TileLoader<D, BMQ, NT> qload, doload;
 	qload.init(a.q.ss, tid);
@@ -204,7 +196,11 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 			int64_t idx = ((int64_t)b * a.Hq + hq) * a.Sq + i;
 			if (tid < BMQ) {
 				x = a.lse[idx];
-				if constexpr (!BIAS) x *= kLog2e;
+				// FOLD: in units of the raw dot product (c1 of them make one log2 unit)
+				if constexpr (FOLD)
+					x *= inv_scale;
+				else if constexpr (!BIAS)
+					x *= kLog2e;
 			} else {
 				x = a.delta[idx];
 			}
@@ -279,6 +275,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		V8 afr[RING];                     // fragments of Q_i / dO_i for the products of A
 		u32x4 cfr[RING];                  // transposed fragments of dO_i / Q_i for the products of C
 		f32x4 lse4[4], del4[4];
+		f32x16 cstart[2];                 // start values of the chains of S and dP (inline-assembly path)
 		float bv[2][BIAS && !BIAS_LDS ? 16 : 1];  // [block parity]: bias values, fetched one stage ahead of their use
 		u32x2 bvr[2][BIAS_LDS ? 4 : 1];           // the same from LDS: [block parity][quad], 4 values of 16 bits
 		const FA2_LDS char* bt = lds_bias + buf * BIAS_BYTES;
@@ -345,10 +342,13 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 			if constexpr (KV_AGPR) {
 				// the chains start from -lse and -delta of the block's rows (accumulator element i
 				// belongs to row 8 (i / 4) + 4 g + i % 4, which is element i % 4 of quarter i / 4)
-				if (j == 0)
-					mfma32_vc(sa, afr[r], kf[ks], __builtin_shufflevector(__builtin_shufflevector(lse4[0], lse4[1], 0, 1, 2, 3, 4, 5, 6, 7), __builtin_shufflevector(lse4[2], lse4[3], 0, 1, 2, 3, 4, 5, 6, 7), 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15));
-				else if (j == 1)
-					mfma32_vc(dpa, afr[r], vf[ks], __builtin_shufflevector(__builtin_shufflevector(del4[0], del4[1], 0, 1, 2, 3, 4, 5, 6, 7), __builtin_shufflevector(del4[2], del4[3], 0, 1, 2, 3, 4, 5, 6, 7), 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15));
+				if (j == 0) {
+					cstart[0] = __builtin_shufflevector(__builtin_shufflevector(lse4[0], lse4[1], 0, 1, 2, 3, 4, 5, 6, 7), __builtin_shufflevector(lse4[2], lse4[3], 0, 1, 2, 3, 4, 5, 6, 7), 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
+					mfma32_vc(sa, afr[r], kf[ks], cstart[0]);
+				} else if (j == 1) {
+					cstart[1] = __builtin_shufflevector(__builtin_shufflevector(del4[0], del4[1], 0, 1, 2, 3, 4, 5, 6, 7), __builtin_shufflevector(del4[2], del4[3], 0, 1, 2, 3, 4, 5, 6, 7), 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
+					mfma32_vc(dpa, afr[r], vf[ks], cstart[1]);
+				}
 				else if (j & 1)
 					mfma32_va<true>(dpa, afr[r], vf[ks]);
 				else
@@ -426,11 +426,14 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		auto micro_B = [&](int qb, int q, int phase, int e0, int e1, const f32x16& sa, const f32x16& dpa, u32x4(&pbo)[2], u32x4(&sbo)[2])
 		                   __attribute__((always_inline)) {
 			if constexpr (FOLD) {
-				// the accumulators already hold S scale log2(e) - lse and dP - delta
+				// the accumulators already hold q.k - lse / (scale log2(e)) and dP - delta
 				if (phase == 0) {
 #pragma unroll
+					for (int e = e0; e < e1; ++e) bx[q][e] = sa[4 * q + e] * c1;
+				} else if (phase == 1) {
+#pragma unroll
 					for (int e = e0; e < e1; ++e) {
-						float p = exp2_fast(sa[4 * q + e]);
+						float p = exp2_fast(bx[q][e]);
 						if constexpr (MASKED) {
 							int row = m0 + 32 * qb + 8 * q + 4 * g + e;
 							bool ok = row < sq_eff && jcol < sk_eff && (!a.causal || jcol <= row + off);
@@ -563,6 +566,14 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 				// bias of the block whose elementwise stage comes next
 				if constexpr (NEXT_B) load_bias_for_slot(k, j);
 				if constexpr (HAS_A) mfma_A(k, j, s[k & 1], dp[k & 1]);
+				// A matrix product reads its C operand while it runs, and the hardware does not hold back a
+				// vector-ALU write to those registers; for the products issued as inline assembly the compiler
+				// does not either.  The start values of the two chains (the only C operands that are not also
+				// the destination) therefore stay allocated until two further products have been issued.
+				if constexpr (HAS_A && KV_AGPR) {
+					if (j == 2) asm volatile("; chain start of S still allocated" ::"v"(cstart[0]));
+					if (j == 3) asm volatile("; chain start of dP still allocated" ::"v"(cstart[1]));
+				}
 				// the vector-ALU work below must not move above the product: for the products
 				// issued as inline assembly that order is what keeps a read of S / dP at least
 				// two matrix products away from the last product of its chain

@@ -21,8 +21,11 @@
 namespace fa2 {
 
 constexpr int kFwdBN = 64;
-// the running row maximum is only raised when exceeded by more than this (log2 units)
+// with bias: the running row maximum is only raised when exceeded by more than this (log2 units)
 constexpr float kRescaleSlack = 8.f;
+// without bias: largest partial row sum of one tile of P = exp2(c1 S - c1 m) taken without looking at
+// the row maximum (fp16 holds values up to 65504)
+constexpr float kFastSum = 16384.f;
 
 // blockIdx.x -> (row tile, q-head, batch).  With xcd_remap the workgroups of
 // one (batch, kv-head) - which share K and V - are kept on one XCD (hardware
@@ -243,30 +246,25 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 		}
 	}
 
-	// Without bias the score only feeds exp2: Q is pre-multiplied by scale * log2(e) and the
-	// chain of S starts from minus the row's running reference instead of 0 (nm16: the value
-	// repeated over the 16 accumulator registers, all of which belong to the lane's row), so
-	// that P = exp2(S accumulator) with no further arithmetic.
+	// Without bias the score only feeds exp2: P = exp2(c1 * q.k - c1 * m) with m the row's running
+	// reference in units of the raw dot product.  The factor c1 = scale * log2(e) is applied to the
+	// fp32 accumulator, as the reference scales the fp32 result of its dot (_forward_triton.py:281).
 	constexpr bool FOLD = !BIAS;
-	if constexpr (FOLD) {
-		const float qc = a.scale * kLog2e;
+	float nmc[QB];  // -c1 * m of the lane's row (0 while the row has seen no key)
+	// The Q fragments must have arrived before the loop over key tiles starts.  Otherwise the
+	// compiler places its waits for these loads (s_waitcnt vmcnt) at their first uses inside the
+	// loop, where the same counter also counts the tile copies in flight: every such wait would
+	// then stall the matrix products until the copies of the NEXT tile have landed.
 #pragma unroll
-		for (int qb = 0; qb < QB; ++qb)
+	for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
-			for (int ks = 0; ks < KS; ++ks) {
-				V8 x = qf[qb][ks];
-				qf[qb][ks] = pack8<T>((float)x[0] * qc, (float)x[1] * qc, (float)x[2] * qc, (float)x[3] * qc, (float)x[4] * qc,
-				                      (float)x[5] * qc, (float)x[6] * qc, (float)x[7] * qc);
-			}
-	}
-	f32x16 nm16[QB];
+		for (int ks = 0; ks < KS; ++ks) asm volatile("; Q fragment present" : "+v"(qf[qb][ks]));
 
 	f32x16 oacc[QB][DB];
 	float mrow[QB], lrow[QB];
 #pragma unroll
 	for (int qb = 0; qb < QB; ++qb) {
-#pragma unroll
-		for (int i = 0; i < 16; ++i) nm16[qb][i] = 0.f;
+		nmc[qb] = 0.f;
 		mrow[qb] = -INFINITY;
 		lrow[qb] = 0.f;
 #pragma unroll
@@ -346,35 +344,36 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 
 		// S^T = K Q^T
 		f32x16 s[KB][QB];
+		auto compute_s = [&]() __attribute__((always_inline)) {
 #pragma unroll
-		for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-			for (int qb = 0; qb < QB; ++qb)
-#pragma unroll
-				for (int i = 0; i < 16; ++i) s[kb][qb][i] = 0.f;
-		__builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-		for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-			for (int kb = 0; kb < KB; ++kb) {
-				V8 kf = *(const FA2_LDS V8*)(kt + koff[ks] + kb * (32 * D * 2));
+			for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
 				for (int qb = 0; qb < QB; ++qb)
-					s[kb][qb] = mfma32(kf, qf[qb][ks], (FOLD && ks == 0) ? nm16[qb] : s[kb][qb]);
-			}
-		// issue order: a few fragment reads ahead, then one read per product, so that the
-		// LDS latency is paid once per tile instead of once per product
-		{
-			constexpr int NR = KS * KB, PF = NR < 8 ? NR : 8;
-			__builtin_amdgcn_sched_group_barrier(0x100, PF, 0);
 #pragma unroll
-			for (int i = 0; i < NR - PF; ++i) {
-				__builtin_amdgcn_sched_group_barrier(0x008, QB, 0);
-				__builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+					for (int i = 0; i < 16; ++i) s[kb][qb][i] = 0.f;
+			__builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+			for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+				for (int kb = 0; kb < KB; ++kb) {
+					V8 kf = *(const FA2_LDS V8*)(kt + koff[ks] + kb * (32 * D * 2));
+#pragma unroll
+					for (int qb = 0; qb < QB; ++qb) s[kb][qb] = mfma32(kf, qf[qb][ks], s[kb][qb]);
+				}
+			// issue order: a few fragment reads ahead, then one read per product, so that the
+			// LDS latency is paid once per tile instead of once per product
+			{
+				constexpr int NR = KS * KB, PF = NR < 8 ? NR : 8;
+				__builtin_amdgcn_sched_group_barrier(0x100, PF, 0);
+#pragma unroll
+				for (int i = 0; i < NR - PF; ++i) {
+					__builtin_amdgcn_sched_group_barrier(0x008, QB, 0);
+					__builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+				}
+				__builtin_amdgcn_sched_group_barrier(0x008, PF * QB, 0);
 			}
-			__builtin_amdgcn_sched_group_barrier(0x008, PF * QB, 0);
-		}
-		__builtin_amdgcn_sched_barrier(0);
+			__builtin_amdgcn_sched_barrier(0);
+		};
 
 		// V fragments for O^T += V^T P^T, fetched in batches of NF; the first batch is in
 		// flight during the softmax, each further one during the products of the previous.
@@ -392,66 +391,145 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 					dst[f * DB + db] = lds_tr_issue_rt<D>(vt + voff[db][0], vt + voff[db][1], BI * FPB + f);
 				}
 		};
-		issue_v(std::integral_constant<int, 0>{}, vfr[0]);
 
-		// online softmax, one query row per lane.  The running reference m of a row is
-		// only raised when some row of the wave exceeds it by more than kRescaleSlack
-		// (log2 units): until then P = exp2(x - m) may grow to 2^slack, which fp32 sums and
-		// 16-bit P hold without loss, and the O accumulators are left alone.
+		// online softmax, one query row per lane
 		V8 pf[QB][BN / 16];
+		compute_s();
+		issue_v(std::integral_constant<int, 0>{}, vfr[0]);
+		// packs P (held in s) to the B operand of the second product, after dropout
+		auto pack_p = [&](int qb) __attribute__((always_inline)) {
+			if constexpr (DROP) {
 #pragma unroll
-		for (int qb = 0; qb < QB; ++qb) {
-			// four independent partial maxima (and, below, partial sums): a chain of dependent
-			// vector-ALU operations pays the full pipeline latency at every link
-			float mx4[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+				for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+					for (int aa = 0; aa < 4; ++aa) {
+						int j4 = (n0 + 32 * kb + 8 * aa + 4 * g) >> 2;
+						u32x4 rnd = philox4x32_10((uint32_t)j4, (uint32_t)qrow[qb], (uint32_t)hl[qb], (uint32_t)b, a.drop_k0, a.drop_k1);
+#pragma unroll
+						for (int e = 0; e < 4; ++e)
+							s[kb][qb][4 * aa + e] = rnd[e] >= a.drop_thr ? s[kb][qb][4 * aa + e] : 0.f;
+					}
+			}
 #pragma unroll
 			for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-				for (int i = 0; i < 16; ++i) {
-					float x = s[kb][qb][i];
-					if constexpr (BIAS) x = __builtin_fmaf(x, c1, bv[kb][qb][i >> 2][i & 3]);
-					if constexpr (MASKED) {
-						int j = n0 + 32 * kb + 8 * (i >> 2) + 4 * g + (i & 3);
-						x = j <= jmax[qb] ? x : -INFINITY;
-					}
-					s[kb][qb][i] = x;
-					mx4[i & 3] = __builtin_fmaxf(mx4[i & 3], x);
+				for (int hf = 0; hf < 2; ++hf) {
+					const f32x16& r = s[kb][qb];
+					pf[qb][2 * kb + hf] = pack8<T>(r[8 * hf + 0], r[8 * hf + 1], r[8 * hf + 2], r[8 * hf + 3], r[8 * hf + 4],
+					                               r[8 * hf + 5], r[8 * hf + 6], r[8 * hf + 7]);
 				}
-			float mx = __builtin_fmaxf(__builtin_fmaxf(mx4[0], mx4[1]), __builtin_fmaxf(mx4[2], mx4[3]));
-			mx = pair_max(mx);
-			float ls4[4] = {0.f, 0.f, 0.f, 0.f};
-			if constexpr (FOLD) {
-				// the accumulators hold x - m (log2 units), mx is the largest of them
-				const bool fresh = mrow[qb] == -INFINITY;  // no key seen so far: any finite maximum becomes the reference
-				if (__builtin_amdgcn_ballot_w64(mx > kRescaleSlack || (fresh && mx > -INFINITY)) != 0) {
-					const float m_old = fresh ? 0.f : mrow[qb];
-					float m_new = __builtin_fmaxf(mrow[qb], m_old + mx);
-					const float m_use = m_new == -INFINITY ? 0.f : m_new;
-					const float shift = m_use - m_old;
-					const float alpha = fresh ? 1.f : exp2_fast(-shift);  // (fresh: l = 0 and O = 0)
-					mrow[qb] = m_new;
-					lrow[qb] *= alpha;
+		};
+		if constexpr (FOLD) {
+			// Fast path (not with dropout): P = exp2(c1 S - c1 m) against the reference m the rows
+			// already have, packed to 16 bits at once - no row maximum, and the scores stay in their
+			// registers.  It stands when every partial row sum of the tile stays below kFastSum (then no
+			// P exceeds it either: 16-bit P and the fp32 sums hold that without loss) and no row meets
+			// its first keys in this tile.  Otherwise (decided for the wave as a whole) the tile takes
+			// the path with the row maximum, from the scores that are still there.
+			constexpr bool FAST = !DROP;
+			float lt[QB];
+			bool slow = true;
+			if constexpr (FAST) {
+				// (a row that meets its first keys here has no reference yet: what the fast path makes of it is discarded)
+				bool over = false;
 #pragma unroll
-					for (int db = 0; db < DB; ++db)
-#pragma unroll
-						for (int i = 0; i < 16; ++i) oacc[qb][db][i] *= alpha;
+				for (int qb = 0; qb < QB; ++qb) {
+					float ls4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
 					for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-						for (int i = 0; i < 16; ++i) s[kb][qb][i] -= shift;
+						for (int hf = 0; hf < 2; ++hf) {
+							float pv[8];
 #pragma unroll
-					for (int i = 0; i < 16; ++i) nm16[qb][i] = -m_use;
+							for (int e = 0; e < 8; ++e) pv[e] = __builtin_fmaf(s[kb][qb][8 * hf + e], c1, nmc[qb]);
+#pragma unroll
+							for (int e = 0; e < 8; ++e) {
+								float p = exp2_fast(pv[e]);
+								if constexpr (MASKED) {
+									int j = n0 + 32 * kb + 8 * (2 * hf + (e >> 2)) + 4 * g + (e & 3);
+									p = j <= jmax[qb] ? p : 0.f;
+								}
+								ls4[e & 3] += p;
+								pv[e] = p;
+							}
+							pf[qb][2 * kb + hf] = pack8<T>(pv[0], pv[1], pv[2], pv[3], pv[4], pv[5], pv[6], pv[7]);
+						}
+					lt[qb] = (ls4[0] + ls4[1]) + (ls4[2] + ls4[3]);
+					// (a NaN sum - from inf or NaN inputs - also takes the other path, which propagates it)
+					over = over || !(lt[qb] <= kFastSum) || (mrow[qb] == -INFINITY && jmax[qb] >= n0);
 				}
+				slow = __builtin_amdgcn_ballot_w64(over) != 0;
+			}
+			if (slow) {
+#pragma unroll
+				for (int qb = 0; qb < QB; ++qb) {
+					// four independent partial maxima (and, below, partial sums): a chain of dependent
+					// vector-ALU operations pays the full pipeline latency at every link
+					float mx4[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+#pragma unroll
+					for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+						for (int i = 0; i < 16; ++i) {
+							float x = s[kb][qb][i];
+							if constexpr (MASKED) {
+								int j = n0 + 32 * kb + 8 * (i >> 2) + 4 * g + (i & 3);
+								x = j <= jmax[qb] ? x : -INFINITY;
+							}
+							s[kb][qb][i] = x;
+							mx4[i & 3] = __builtin_fmaxf(mx4[i & 3], x);
+						}
+					float mx = __builtin_fmaxf(__builtin_fmaxf(mx4[0], mx4[1]), __builtin_fmaxf(mx4[2], mx4[3]));
+					mx = pair_max(mx);
+					// the row maximum becomes the reference whenever it exceeds it
+					if (mx > mrow[qb]) {
+						// (first keys of the row: l = 0 and O = 0, alpha = exp2(-inf) = 0 leaves them so)
+						const float alpha = exp2_fast((mrow[qb] - mx) * c1);
+						mrow[qb] = mx;
+						nmc[qb] = -mx * c1;
+						lrow[qb] *= alpha;
+#pragma unroll
+						for (int db = 0; db < DB; ++db)
+#pragma unroll
+							for (int i = 0; i < 16; ++i) oacc[qb][db][i] *= alpha;
+					}
+					float ls4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+					for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+						for (int i = 0; i < 16; ++i) {
+							float p = exp2_fast(__builtin_fmaf(s[kb][qb][i], c1, nmc[qb]));
+							ls4[i & 3] += p;
+							s[kb][qb][i] = p;
+						}
+					lt[qb] = (ls4[0] + ls4[1]) + (ls4[2] + ls4[3]);
+					pack_p(qb);
+				}
+			}
+#pragma unroll
+			for (int qb = 0; qb < QB; ++qb) lrow[qb] += lt[qb];
+		} else {
+#pragma unroll
+			for (int qb = 0; qb < QB; ++qb) {
+				float mx4[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
 #pragma unroll
 				for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
 					for (int i = 0; i < 16; ++i) {
-						float p = exp2_fast(s[kb][qb][i]);
-						ls4[i & 3] += p;
-						s[kb][qb][i] = p;
+						float x = __builtin_fmaf(s[kb][qb][i], c1, bv[kb][qb][i >> 2][i & 3]);
+						if constexpr (MASKED) {
+							int j = n0 + 32 * kb + 8 * (i >> 2) + 4 * g + (i & 3);
+							x = j <= jmax[qb] ? x : -INFINITY;
+						}
+						s[kb][qb][i] = x;
+						mx4[i & 3] = __builtin_fmaxf(mx4[i & 3], x);
 					}
-			} else {
-				// natural units with bias
+				float mx = __builtin_fmaxf(__builtin_fmaxf(mx4[0], mx4[1]), __builtin_fmaxf(mx4[2], mx4[3]));
+				mx = pair_max(mx);
+				float ls4[4] = {0.f, 0.f, 0.f, 0.f};
+				// natural units with bias.  The running reference m of a row is only raised when some
+				// row of the wave exceeds it by more than kRescaleSlack (log2 units): until then
+				// P = exp2(x - m) may grow to 2^slack, which fp32 sums and 16-bit P hold without loss,
+				// and the O accumulators are left alone.
 				const float slack = kRescaleSlack * kLn2;
 				if (__builtin_amdgcn_ballot_w64(mx > mrow[qb] + slack) != 0) {
 					float m_new = __builtin_fmaxf(mrow[qb], mx);
@@ -473,28 +551,9 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 						ls4[i & 3] += p;
 						s[kb][qb][i] = p;
 					}
+				lrow[qb] += (ls4[0] + ls4[1]) + (ls4[2] + ls4[3]);
+				pack_p(qb);
 			}
-			lrow[qb] += (ls4[0] + ls4[1]) + (ls4[2] + ls4[3]);
-			if constexpr (DROP) {
-#pragma unroll
-				for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-					for (int aa = 0; aa < 4; ++aa) {
-						int j4 = (n0 + 32 * kb + 8 * aa + 4 * g) >> 2;
-						u32x4 rnd = philox4x32_10((uint32_t)j4, (uint32_t)qrow[qb], (uint32_t)hl[qb], (uint32_t)b, a.drop_k0, a.drop_k1);
-#pragma unroll
-						for (int e = 0; e < 4; ++e)
-							s[kb][qb][4 * aa + e] = rnd[e] >= a.drop_thr ? s[kb][qb][4 * aa + e] : 0.f;
-					}
-			}
-#pragma unroll
-			for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-				for (int hf = 0; hf < 2; ++hf) {
-					const f32x16& r = s[kb][qb];
-					pf[qb][2 * kb + hf] = pack8<T>(r[8 * hf + 0], r[8 * hf + 1], r[8 * hf + 2], r[8 * hf + 3], r[8 * hf + 4],
-					                               r[8 * hf + 5], r[8 * hf + 6], r[8 * hf + 7]);
-				}
 		}
 
 		// O^T += V^T P^T
@@ -509,10 +568,21 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 					for (int qb = 0; qb < QB; ++qb)
 						oacc[qb][db] = mfma32(as_frag<T>(vfr[BI & 1][f * DB + db]), pf[qb][BI * FPB + f], oacc[qb][db]);
 		};
+		__builtin_amdgcn_sched_barrier(0);
 		pv_batch(std::integral_constant<int, 0>{});
 		if constexpr (NBATCH > 1) pv_batch(std::integral_constant<int, 1>{});
 		if constexpr (NBATCH > 2) pv_batch(std::integral_constant<int, 2>{});
 		if constexpr (NBATCH > 3) pv_batch(std::integral_constant<int, 3>{});
+		// issue order: every product of a batch but the last is followed by the two transposed reads
+		// of one fragment of the next batch (left to itself the compiler's order, and with it the
+		// kernel's duration, changes with unrelated edits)
+#pragma unroll
+		for (int i = 0; i < (NBATCH - 1) * NF; ++i) {
+			__builtin_amdgcn_sched_group_barrier(0x008, QB, 0);
+			__builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+		}
+		__builtin_amdgcn_sched_group_barrier(0x008, NF * QB, 0);
+		__builtin_amdgcn_sched_barrier(0);
 		static_assert(NBATCH <= 4, "");
 	};
 
@@ -575,7 +645,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 					}
 				if (g == 0) {
 					float lse = -INFINITY;
-					if (lt > 0.f) lse = BIAS ? mrow[qb] + log2_fast(lt) * kLn2 : (mrow[qb] + log2_fast(lt)) * kLn2;
+					if (lt > 0.f) lse = BIAS ? mrow[qb] + log2_fast(lt) * kLn2 : (mrow[qb] * c1 + log2_fast(lt)) * kLn2;
 					a.lse_part[row] = lse;
 				}
 			}
@@ -595,7 +665,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 			if (g == 0) {
 				float lse;
 				if (lt > 0.f)
-					lse = BIAS ? mrow[qb] + log2_fast(lt) * kLn2 : (mrow[qb] + log2_fast(lt)) * kLn2;
+					lse = BIAS ? mrow[qb] + log2_fast(lt) * kLn2 : (mrow[qb] * c1 + log2_fast(lt)) * kLn2;
 				else
 					lse = -INFINITY;
 				a.lse[((int64_t)b * a.Hq + h) * a.Sq + i] = lse;

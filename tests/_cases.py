@@ -11,11 +11,14 @@ TOL_GRAD_REL_L2 = 1e-2
 TOL_LSE = 1e-2
 
 
-def make_inputs(B, Sq, Sk, Hq, Hkv, D, dtype, seed=0, bias_shape=None, scale=0.5, bias_dtype=None):
-	"""Seeded CPU tensors, already rounded to `dtype`, so the oracle consumes the kernel's exact inputs."""
+def make_inputs(B, Sq, Sk, Hq, Hkv, D, dtype, seed=0, bias_shape=None, scale=0.5, bias_dtype=None, qk_scale=None):
+	"""Seeded CPU tensors, already rounded to `dtype`, so the oracle consumes the kernel's exact inputs.
+	qk_scale: standard deviation of q and k when it differs from that of v (the scores of a head of
+	dim D then have a standard deviation of qk_scale^2 at the default softmax scale)."""
 	g = torch.Generator().manual_seed(seed)
-	q = (torch.randn(B, Sq, Hq, D, generator=g) * scale).to(dtype)
-	k = (torch.randn(B, Sk, Hkv, D, generator=g) * scale).to(dtype)
+	qs = scale if qk_scale is None else qk_scale
+	q = (torch.randn(B, Sq, Hq, D, generator=g) * qs).to(dtype)
+	k = (torch.randn(B, Sk, Hkv, D, generator=g) * qs).to(dtype)
 	v = (torch.randn(B, Sk, Hkv, D, generator=g) * scale).to(dtype)
 	do = torch.randn(B, Sq, Hq, D, generator=g).to(dtype)
 	bias = None

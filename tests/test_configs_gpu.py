@@ -126,6 +126,6 @@ def test_c5_dropout_wide_heads_bf16_causal_fwd_bwd():
 	grads = op.bwd(q, k, v, o, lse, do, None, None, None, 0.1, True, 42)
 	for b, h in ((0, 0), (7, 15)):
 		_check_group(q, k, v, do, o, lse, grads, b, h, 1, dtype, causal=True, p_drop=0.1, seed=42)
-	# LSE does not depend on dropout
+	# LSE does not depend on dropout (up to fp32 rounding: the two variants of the kernel hold different running references)
 	_, lse0 = op.fwd(q, k, v, causal=True)
-	assert torch.equal(lse, lse0)
+	assert torch.allclose(lse, lse0, rtol=0, atol=1e-5)

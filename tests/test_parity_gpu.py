@@ -26,8 +26,8 @@ def _dev(t):
 
 
 def _run_case(B, Sq, Sk, Hq, Hkv, D, dtype, causal=False, bias_shape=None, p=0.0, seed=0, seqlens=None, scale=None,
-              bias_dtype=None, data_seed=0):
-	q, k, v, do, bias = make_inputs(B, Sq, Sk, Hq, Hkv, D, dtype, data_seed, bias_shape, bias_dtype=bias_dtype)
+              bias_dtype=None, data_seed=0, qk_scale=None):
+	q, k, v, do, bias = make_inputs(B, Sq, Sk, Hq, Hkv, D, dtype, data_seed, bias_shape, bias_dtype=bias_dtype, qk_scale=qk_scale)
 	sl = None if seqlens is None else torch.tensor(seqlens, dtype=torch.int32)
 	kw = dict(causal=causal, p_drop=p, seed=seed, seqlens=seqlens, scale=scale)
 	o_ref, lse_ref = O.attention_fwd(f64(q), f64(k), f64(v), f64(bias), **kw)
@@ -45,6 +45,21 @@ def _run_case(B, Sq, Sk, Hq, Hkv, D, dtype, causal=False, bias_shape=None, p=0.0
 @pytest.mark.parametrize("causal", [False, True])
 def test_basic_shapes(dtype, D, causal):
 	_run_case(2, 320, 320, 4, 2, D, dtype, causal=causal)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("qk_scale,score_range", [(2.1, 20), (4.2, 80)])
+def test_large_logits(dtype, qk_scale, score_range):
+	"""Scores of realistic and of extreme magnitude (within about +-20 and +-80; the other cases stay within +-5):
+	the softmax scale is applied to the fp32 result of q.k as the reference does (_forward_triton.py:281), so the
+	tolerances hold at any magnitude.  v keeps its usual size, so that O stays of order 1."""
+	q, k, *_ = make_inputs(2, 384, 384, 4, 2, 128, dtype, qk_scale=qk_scale)
+	sc = torch.einsum("bihd,bjhd->bhij", q.float(), k.float().repeat_interleave(2, dim=2)) / 128**0.5
+	assert 0.7 * score_range <= sc.abs().max().item() <= 1.3 * score_range
+	_run_case(2, 384, 384, 4, 2, 128, dtype, causal=True, qk_scale=qk_scale)
+	_run_case(1, 200, 333, 4, 4, 64, dtype, causal=False, qk_scale=qk_scale, data_seed=1)
+	_run_case(1, 160, 160, 2, 1, 256, dtype, causal=True, qk_scale=qk_scale, data_seed=2)
+	_run_case(1, 160, 160, 2, 2, 128, dtype, causal=True, qk_scale=qk_scale, p=0.1, seed=5, data_seed=3)
 
 
 @pytest.mark.parametrize(
