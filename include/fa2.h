@@ -35,7 +35,7 @@ enum { FA2_FP16 = 1, FA2_BF16 = 2, FA2_FP32 = 3 /* bias only */ };
 /* Return codes. 0 = success, negative = error; nothing is launched on error. */
 enum {
 	FA2_OK = 0,
-	FA2_EINVAL_STRUCT = -1,   /* NULL params or struct_size too small            */
+	FA2_EINVAL_STRUCT = -1,   /* NULL params or struct_size < FA2_PARAMS_SIZE_V1  */
 	FA2_EINVAL_DTYPE = -2,    /* q/k/v dtype not fp16/bf16 (_forward_triton.py:494-495) */
 	FA2_EINVAL_SHAPE = -3,    /* non-positive dimension, or scale not finite and > 0 */
 	FA2_EINVAL_HEADS = -4,    /* Hq % Hkv != 0 (flash_attention.py:189-193)      */
@@ -61,7 +61,8 @@ typedef struct fa2_tensor {
 } fa2_tensor;
 
 typedef struct fa2_params {
-	uint32_t struct_size;   /* = sizeof(fa2_params), checked first        */
+	uint32_t struct_size;   /* = sizeof(fa2_params) of the header the caller was built
+	                           with (>= FA2_PARAMS_SIZE_V1), checked first */
 	int32_t dtype;          /* FA2_FP16 | FA2_BF16 for q,k,v,o,dO,dq,dk,dv */
 	int32_t B, Sq, Sk, Hq, Hkv, D;
 	int32_t causal;         /* bottom-right aligned: j <= i + Sk - Sq
@@ -98,7 +99,21 @@ typedef struct fa2_params {
 	 * fa2_fwd_scratch_bytes().  256-byte aligned. */
 	void* scratch;
 	uint64_t scratch_bytes;
+
+	/* --- fields added after the first version of this header (FA2_PARAMS_SIZE_V1 bytes);
+	 *     a caller that passes the shorter struct_size gets zeros for them --- */
+
+	/* Optional: the Philox key as a 64-bit value in DEVICE memory (8-byte aligned).  When
+	 * non-NULL the kernels read it there and `seed` is ignored, so the key can be an
+	 * ordinary runtime operand of the caller's graph - the reference passes its
+	 * dropout_seed to the custom call as an operand, not as a compile-time constant
+	 * (_forward_triton.py:553, _flash_attention.py:91-92) - and changing it needs neither a
+	 * new parameter block nor, under XLA, a new executable.                              */
+	const uint64_t* seed_dev;
 } fa2_params;
+
+/* sizeof(fa2_params) in the first version of this header: up to and including scratch_bytes */
+#define FA2_PARAMS_SIZE_V1 ((uint32_t)offsetof(fa2_params, seed_dev))
 
 /* O = softmax(scale q k^T + bias, masked) v, with dropout; writes o and lse.
  * Replaces the `_attn_fwd` custom call (_forward_triton.py:547-588). */
@@ -146,7 +161,7 @@ int fa2_bwd_static(const fa2_params* p, void* hip_stream);
 /* keep[b,h,i,j] (uint8, contiguous [B,Hq,Sq,Sk]) of the dropout mask the
  * kernels apply for (seed, p_drop); for validation against the Philox
  * definition.  Counterpart of `tl.rand(seed, offs) > p`
- * (_forward_triton.py:140-143). Uses B, Hq, Sq, Sk, p_drop, seed only. */
+ * (_forward_triton.py:140-143). Uses B, Hq, Sq, Sk, p_drop, seed / seed_dev only. */
 int fa2_dropout_mask(const fa2_params* p, uint8_t* keep, void* hip_stream);
 
 /* Validate params exactly as fa2_fwd / fa2_bwd would, without launching

@@ -20,6 +20,17 @@ using fa2::KTensor;
 
 bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
+// Parameter blocks of earlier versions of the header are shorter (struct_size says which): they are
+// completed with zeros.  Returns NULL for a NULL block or one shorter than the first version.
+const fa2_params* complete(const fa2_params* p, fa2_params& local) {
+	if (!p || p->struct_size < FA2_PARAMS_SIZE_V1) return nullptr;
+	if (p->struct_size >= sizeof(fa2_params)) return p;
+	memset(&local, 0, sizeof(local));
+	memcpy(&local, p, p->struct_size);
+	local.struct_size = sizeof(fa2_params);
+	return &local;
+}
+
 int check_tensor(const fa2_tensor& t, bool required) {
 	if (!t.ptr) return required ? FA2_EINVAL_PTR : FA2_OK;
 	if (!aligned16(t.ptr)) return FA2_EINVAL_PTR;
@@ -43,7 +54,8 @@ KTensor conv(const fa2_tensor& t) {
 
 // own_scratch: the backward brings its scratch itself (fa2_bwd_static), p->scratch is not looked at
 int validate(const fa2_params* p, int which, bool own_scratch = false) {
-	if (!p || p->struct_size < sizeof(fa2_params)) return FA2_EINVAL_STRUCT;
+	if (!p) return FA2_EINVAL_STRUCT;
+	if (p->seed_dev && ((uintptr_t)p->seed_dev & 7)) return FA2_EINVAL_PTR;
 	if (p->dtype != FA2_FP16 && p->dtype != FA2_BF16) return FA2_EINVAL_DTYPE;
 	if (p->B <= 0 || p->Sq <= 0 || p->Sk <= 0 || p->Hq <= 0 || p->Hkv <= 0 || p->D <= 0) return FA2_EINVAL_SHAPE;
 	if (p->Hq % p->Hkv) return FA2_EINVAL_HEADS;
@@ -122,6 +134,7 @@ void fill(const fa2_params* p, KArgs& a) {
 	a.scale = p->scale;
 	a.drop_k0 = (uint32_t)(p->seed & 0xFFFFFFFFull);
 	a.drop_k1 = (uint32_t)(p->seed >> 32);
+	a.seed_dev = (const uint32_t*)p->seed_dev;  // little-endian: low word first
 	a.drop_thr = drop_threshold(p->p_drop);
 	a.drop_inv_keep = 1.0f / (1.0f - p->p_drop);
 }
@@ -156,10 +169,13 @@ hipError_t launch_bwd(int dtype, int D, bool bias, bool drop, KArgs& a, hipStrea
 
 extern "C" {
 
-int fa2_validate(const fa2_params* p, int which) { return validate(p, which ? 1 : 0); }
+int fa2_validate(const fa2_params* p, int which) {
+	fa2_params lp;
+	return validate(complete(p, lp), which ? 1 : 0);
+}
 
 size_t fa2_bwd_scratch_bytes(const fa2_params* p) {
-	if (!p || p->struct_size < sizeof(fa2_params)) return 0;
+	if (!p || p->struct_size < FA2_PARAMS_SIZE_V1) return 0;
 	if (p->B <= 0 || p->Hq <= 0 || p->Sq <= 0) return 0;
 	// delta [B, Hq, Sq] fp32, rounded up to 256 bytes
 	size_t n = (size_t)p->B * (size_t)p->Hq * (size_t)p->Sq * sizeof(float);
@@ -189,7 +205,7 @@ static int fwd_split_plan(const fa2_params* p, int* split_len) {
 }
 
 size_t fa2_fwd_scratch_bytes(const fa2_params* p) {
-	if (!p || p->struct_size < sizeof(fa2_params)) return 0;
+	if (!p || p->struct_size < FA2_PARAMS_SIZE_V1) return 0;
 	if (p->B <= 0 || p->Hq <= 0 || p->Sq <= 0 || p->Sk <= 0 || p->D <= 0) return 0;
 	int len;
 	int n = fwd_split_plan(p, &len);
@@ -199,6 +215,8 @@ size_t fa2_fwd_scratch_bytes(const fa2_params* p) {
 }
 
 int fa2_fwd(const fa2_params* p, void* hip_stream) {
+	fa2_params lp;
+	p = complete(p, lp);
 	int rc = validate(p, 0);
 	if (rc) return rc;
 	KArgs a;
@@ -232,6 +250,8 @@ static int bwd_launch(const fa2_params* p, void* hip_stream, int stages, void* s
 }
 
 int fa2_bwd_stages(const fa2_params* p, void* hip_stream, int stages) {
+	fa2_params lp;
+	p = complete(p, lp);
 	int rc = validate(p, 1);
 	if (rc) return rc;
 	return bwd_launch(p, hip_stream, stages, p->scratch);
@@ -255,6 +275,8 @@ static int static_scratch_ptr(void** out) {
 }
 
 int fa2_bwd_static(const fa2_params* p, void* hip_stream) {
+	fa2_params lp;
+	p = complete(p, lp);
 	int rc = validate(p, 1, /*own_scratch=*/true);
 	if (rc) return rc;
 	void* ptr = nullptr;
@@ -264,19 +286,23 @@ int fa2_bwd_static(const fa2_params* p, void* hip_stream) {
 }
 
 int fa2_dropout_mask(const fa2_params* p, uint8_t* keep, void* hip_stream) {
-	if (!p || p->struct_size < sizeof(fa2_params)) return FA2_EINVAL_STRUCT;
+	fa2_params lp;
+	p = complete(p, lp);
+	if (!p) return FA2_EINVAL_STRUCT;
+	if (p->seed_dev && ((uintptr_t)p->seed_dev & 7)) return FA2_EINVAL_PTR;
 	if (p->B <= 0 || p->Sq <= 0 || p->Sk <= 0 || p->Hq <= 0) return FA2_EINVAL_SHAPE;
 	if (!(p->p_drop >= 0.f && p->p_drop < 1.f)) return FA2_EINVAL_DROPOUT;
 	if (!keep) return FA2_EINVAL_PTR;
 	hipError_t e = fa2::launch_dropout_mask(keep, p->B, p->Hq, p->Sq, p->Sk, (uint32_t)(p->seed & 0xFFFFFFFFull),
-	                                        (uint32_t)(p->seed >> 32), drop_threshold(p->p_drop), (hipStream_t)hip_stream);
+	                                        (uint32_t)(p->seed >> 32), drop_threshold(p->p_drop), (const uint32_t*)p->seed_dev,
+	                                        (hipStream_t)hip_stream);
 	return e == hipSuccess ? FA2_OK : FA2_EHIP;
 }
 
 const char* fa2_strerror(int code) {
 	switch (code) {
 		case FA2_OK: return "ok";
-		case FA2_EINVAL_STRUCT: return "params is NULL or struct_size is smaller than sizeof(fa2_params)";
+		case FA2_EINVAL_STRUCT: return "params is NULL or struct_size is smaller than the first version of fa2_params";
 		case FA2_EINVAL_DTYPE: return "Only support fp16 and bf16";
 		case FA2_EINVAL_SHAPE: return "dimensions must be positive and the softmax scale finite and positive";
 		case FA2_EINVAL_HEADS: return "query heads must be divisible by key/value heads";

@@ -93,6 +93,14 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
 	const int g = lane >> 5, c = lane & 31;
 	const int r = a.Hq / a.Hkv;
+	// dropout key: from the parameter block, or from device memory when the caller keeps it there
+	uint32_t drop_k0 = a.drop_k0, drop_k1 = a.drop_k1;
+	if constexpr (DROP) {
+		if (a.seed_dev) {
+			drop_k0 = a.seed_dev[0];
+			drop_k1 = a.seed_dev[1];
+		}
+	}
 
 	// blockIdx.x -> (key tile, kv head, batch); key tiles of one (b, kv head) stay on one XCD
 	int nt, hk, b;
@@ -403,13 +411,13 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 					cs[1] = (uint32_t)(m0 + 32 * qb + 8 * q + 4 * g + (c & 3));
 					cs[2] = (uint32_t)hq;
 					cs[3] = (uint32_t)b;
-					philox4x32_rounds<0, 3>(cs, a.drop_k0, a.drop_k1);
+					philox4x32_rounds<0, 3>(cs, drop_k0, drop_k1);
 				} else if (part == 1) {
-					philox4x32_rounds<3, 6>(cs, a.drop_k0, a.drop_k1);
+					philox4x32_rounds<3, 6>(cs, drop_k0, drop_k1);
 				} else if (part == 2) {
-					philox4x32_rounds<6, 8>(cs, a.drop_k0, a.drop_k1);
+					philox4x32_rounds<6, 8>(cs, drop_k0, drop_k1);
 				} else {
-					philox4x32_rounds<8, 10>(cs, a.drop_k0, a.drop_k1);
+					philox4x32_rounds<8, 10>(cs, drop_k0, drop_k1);
 					// bit t = key (jcol & ~3) + t of this lane's row is kept
 					uint32_t mine = (cs[0] >= a.drop_thr ? 1u : 0u) | (cs[1] >= a.drop_thr ? 2u : 0u) | (cs[2] >= a.drop_thr ? 4u : 0u) |
 					                (cs[3] >= a.drop_thr ? 8u : 0u);
@@ -723,6 +731,13 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 	const int hk = h / (a.Hq / a.Hkv);
 	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
 	const int g = lane >> 5, c = lane & 31;
+	uint32_t drop_k0 = a.drop_k0, drop_k1 = a.drop_k1;
+	if constexpr (DROP) {
+		if (a.seed_dev) {
+			drop_k0 = a.seed_dev[0];
+			drop_k1 = a.seed_dev[1];
+		}
+	}
 
 	int sq_eff = a.Sq, sk_eff = a.Sk;
 	if (a.seqlens) {
@@ -944,7 +959,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 					u32x4 rnd;
 					if constexpr (DROP) {
 						int j4 = (n0 + 32 * kb + 8 * aa + 4 * g) >> 2;
-						rnd = philox4x32_10((uint32_t)j4, (uint32_t)qrow[qb], (uint32_t)h, (uint32_t)b, a.drop_k0, a.drop_k1);
+						rnd = philox4x32_10((uint32_t)j4, (uint32_t)qrow[qb], (uint32_t)h, (uint32_t)b, drop_k0, drop_k1);
 					}
 #pragma unroll
 					for (int e = 0; e < 4; ++e) {

@@ -9,7 +9,11 @@ namespace fa2 {
 
 // one thread = four consecutive keys of one (b, h, i)
 __global__ __launch_bounds__(256) void dropout_mask_kernel(uint8_t* keep, int B, int H, int Sq, int Sk, uint32_t k0,
-                                                            uint32_t k1, uint32_t thr) {
+                                                            uint32_t k1, uint32_t thr, const uint32_t* seed_dev) {
+	if (seed_dev) {
+		k0 = seed_dev[0];
+		k1 = seed_dev[1];
+	}
 	int nj4 = (Sk + 3) >> 2;
 	int64_t total = (int64_t)B * H * Sq * nj4;
 	for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
@@ -30,11 +34,11 @@ __global__ __launch_bounds__(256) void dropout_mask_kernel(uint8_t* keep, int B,
 }
 
 hipError_t launch_dropout_mask(uint8_t* keep, int B, int H, int Sq, int Sk, uint32_t k0, uint32_t k1, uint32_t thr,
-                               hipStream_t s) {
+                               const uint32_t* seed_dev, hipStream_t s) {
 	int64_t total = (int64_t)B * H * Sq * ((Sk + 3) / 4);
 	int64_t blocks = (total + 255) / 256;
 	if (blocks > 65536) blocks = 65536;
-	hipLaunchKernelGGL(dropout_mask_kernel, dim3((unsigned)blocks), dim3(256), 0, s, keep, B, H, Sq, Sk, k0, k1, thr);
+	hipLaunchKernelGGL(dropout_mask_kernel, dim3((unsigned)blocks), dim3(256), 0, s, keep, B, H, Sq, Sk, k0, k1, thr, seed_dev);
 	return hipGetLastError();
 }
 

@@ -143,6 +143,14 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 	const int hk = h / (a.Hq / a.Hkv);
 	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
 	const int g = lane >> 5, c = lane & 31;
+	// dropout key: from the parameter block, or from device memory when the caller keeps it there
+	uint32_t drop_k0 = a.drop_k0, drop_k1 = a.drop_k1;
+	if constexpr (DROP) {
+		if (a.seed_dev) {
+			drop_k0 = a.seed_dev[0];
+			drop_k1 = a.seed_dev[1];
+		}
+	}
 
 	int sq_eff = a.Sq, sk_eff = a.Sk;
 	if (a.seqlens) {
@@ -404,7 +412,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 #pragma unroll
 					for (int aa = 0; aa < 4; ++aa) {
 						int j4 = (n0 + 32 * kb + 8 * aa + 4 * g) >> 2;
-						u32x4 rnd = philox4x32_10((uint32_t)j4, (uint32_t)qrow[qb], (uint32_t)hl[qb], (uint32_t)b, a.drop_k0, a.drop_k1);
+						u32x4 rnd = philox4x32_10((uint32_t)j4, (uint32_t)qrow[qb], (uint32_t)hl[qb], (uint32_t)b, drop_k0, drop_k1);
 #pragma unroll
 						for (int e = 0; e < 4; ++e)
 							s[kb][qb][4 * aa + e] = rnd[e] >= a.drop_thr ? s[kb][qb][4 * aa + e] : 0.f;

@@ -27,6 +27,8 @@ struct KArgs {
 	int causal;
 	float scale;
 	uint32_t drop_k0, drop_k1, drop_thr;
+	const uint32_t* seed_dev;  // when set: the Philox key (low word, high word) is read from device memory instead
+
 	float drop_inv_keep;
 	int mtiles;      // number of row tiles of the launched kernel
 	int xcd_remap;   // 1: group-major placement of workgroups on the 8 XCDs
@@ -44,7 +46,7 @@ struct KArgs {
 hipError_t launch_fwd(int dtype, int D, bool bias, bool drop, KArgs& a, hipStream_t s);
 hipError_t launch_bwd(int dtype, int D, bool bias, bool drop, KArgs& a, hipStream_t s);
 hipError_t launch_dropout_mask(uint8_t* keep, int B, int H, int Sq, int Sk, uint32_t k0, uint32_t k1, uint32_t thr,
-                               hipStream_t s);
+                               const uint32_t* seed_dev, hipStream_t s);
 
 // Per-(dtype, D) translation units provide these.
 #define FA2_DECL_FWD(TAG, DD) hipError_t launch_fwd_##TAG##_##DD(bool bias, bool drop, KArgs& a, hipStream_t s);

@@ -12,9 +12,12 @@
 // `make ffi XLA_FFI_INCLUDE=<dir>` and is not part of the default build.
 //
 // Operand convention (absent optional operands are passed as 0-element buffers):
-//   fa2_fwd_ffi : args q, k, v, bias, seqlens        rets o, lse, scratch
-//   fa2_bwd_ffi : args q, k, v, bias, seqlens, o, lse, dout   rets dq, dk, dv, scratch
-//   attrs (both): scale f32, dropout_p f32, causal bool, seed i64, bias_group bool
+//   fa2_fwd_ffi : args q, k, v, bias, seqlens, seed        rets o, lse, scratch
+//   fa2_bwd_ffi : args q, k, v, bias, seqlens, seed, o, lse, dout   rets dq, dk, dv, scratch
+//   attrs (both): scale f32, dropout_p f32, causal bool, bias_group bool
+// The dropout seed is an OPERAND (8 bytes on the device: u32[2] low word first, or one 64-bit
+// integer), as in the reference, whose custom call takes dropout_seed as an operand
+// (_forward_triton.py:553): a new seed then needs no new executable and the seed may be traced.
 // All tensors are dense row-major as XLA lays them out: q/o/dout/dq [B,Sq,Hq,D],
 // k/v/dk/dv [B,Sk,Hkv,D], bias [B|1, H|1, Sq, Sk], lse [B,Hq,Sq] f32,
 // scratch u8: fa2_bwd_scratch_bytes for the backward, fa2_fwd_scratch_bytes (or any smaller size: no split) for the forward.
@@ -48,7 +51,7 @@ fa2_tensor dense4(void* ptr, ffi::Span<const int64_t> d) {
 }
 
 ffi::Error fill_common(fa2_params& p, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::AnyBuffer v, ffi::AnyBuffer bias,
-                       ffi::AnyBuffer seqlens, float scale, float dropout_p, bool causal, int64_t seed, bool bias_group) {
+                       ffi::AnyBuffer seqlens, ffi::AnyBuffer seed, float scale, float dropout_p, bool causal, bool bias_group) {
 	std::memset(&p, 0, sizeof(p));
 	p.struct_size = sizeof(p);
 	auto qd = q.dimensions(), kd = k.dimensions();
@@ -64,7 +67,8 @@ ffi::Error fill_common(fa2_params& p, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::A
 	p.causal = causal ? 1 : 0;
 	p.scale = scale;
 	p.p_drop = dropout_p;
-	p.seed = (uint64_t)seed;
+	if (seed.size_bytes() != 8) return ffi::Error(ffi::ErrorCode::kInvalidArgument, "seed must hold 8 bytes (u32[2] or one 64-bit integer)");
+	p.seed_dev = (const uint64_t*)seed.untyped_data();
 	p.q = dense4(q.untyped_data(), qd);
 	p.k = dense4(k.untyped_data(), kd);
 	p.v = dense4(v.untyped_data(), v.dimensions());
@@ -88,11 +92,10 @@ ffi::Error to_error(int rc) {
 }
 
 ffi::Error FwdImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::AnyBuffer v, ffi::AnyBuffer bias,
-                   ffi::AnyBuffer seqlens, ffi::Result<ffi::AnyBuffer> o, ffi::Result<ffi::AnyBuffer> lse,
-                   ffi::Result<ffi::AnyBuffer> scratch, float scale, float dropout_p, bool causal, int64_t seed,
-                   bool bias_group) {
+                   ffi::AnyBuffer seqlens, ffi::AnyBuffer seed, ffi::Result<ffi::AnyBuffer> o, ffi::Result<ffi::AnyBuffer> lse,
+                   ffi::Result<ffi::AnyBuffer> scratch, float scale, float dropout_p, bool causal, bool bias_group) {
 	fa2_params p;
-	if (auto e = fill_common(p, q, k, v, bias, seqlens, scale, dropout_p, causal, seed, bias_group); e.failure()) return e;
+	if (auto e = fill_common(p, q, k, v, bias, seqlens, seed, scale, dropout_p, causal, bias_group); e.failure()) return e;
 	p.o = dense4(o->untyped_data(), q.dimensions());
 	p.lse = (float*)lse->untyped_data();
 	// optional: with fa2_fwd_scratch_bytes() of scratch a short query is split over key ranges
@@ -102,12 +105,11 @@ ffi::Error FwdImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::
 }
 
 ffi::Error BwdImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::AnyBuffer v, ffi::AnyBuffer bias,
-                   ffi::AnyBuffer seqlens, ffi::AnyBuffer o, ffi::AnyBuffer lse, ffi::AnyBuffer dout,
+                   ffi::AnyBuffer seqlens, ffi::AnyBuffer seed, ffi::AnyBuffer o, ffi::AnyBuffer lse, ffi::AnyBuffer dout,
                    ffi::Result<ffi::AnyBuffer> dq, ffi::Result<ffi::AnyBuffer> dk, ffi::Result<ffi::AnyBuffer> dv,
-                   ffi::Result<ffi::AnyBuffer> scratch, float scale, float dropout_p, bool causal, int64_t seed,
-                   bool bias_group) {
+                   ffi::Result<ffi::AnyBuffer> scratch, float scale, float dropout_p, bool causal, bool bias_group) {
 	fa2_params p;
-	if (auto e = fill_common(p, q, k, v, bias, seqlens, scale, dropout_p, causal, seed, bias_group); e.failure()) return e;
+	if (auto e = fill_common(p, q, k, v, bias, seqlens, seed, scale, dropout_p, causal, bias_group); e.failure()) return e;
 	p.o = dense4(o.untyped_data(), q.dimensions());
 	p.lse = (float*)lse.untyped_data();
 	p.dout = dense4(dout.untyped_data(), q.dimensions());
@@ -119,7 +121,7 @@ ffi::Error BwdImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::
 	return to_error(fa2_bwd(&p, stream));
 }
 
-ffi::Error DropoutMaskImpl(hipStream_t stream, ffi::Result<ffi::AnyBuffer> keep, float dropout_p, int64_t seed) {
+ffi::Error DropoutMaskImpl(hipStream_t stream, ffi::AnyBuffer seed, ffi::Result<ffi::AnyBuffer> keep, float dropout_p) {
 	auto d = keep->dimensions();  // [B, H, Sq, Sk] u8
 	if (d.size() != 4) return ffi::Error(ffi::ErrorCode::kInvalidArgument, "keep must be [B, H, Sq, Sk]");
 	fa2_params p;
@@ -130,7 +132,8 @@ ffi::Error DropoutMaskImpl(hipStream_t stream, ffi::Result<ffi::AnyBuffer> keep,
 	p.Sq = (int32_t)d[2];
 	p.Sk = (int32_t)d[3];
 	p.p_drop = dropout_p;
-	p.seed = (uint64_t)seed;
+	if (seed.size_bytes() != 8) return ffi::Error(ffi::ErrorCode::kInvalidArgument, "seed must hold 8 bytes (u32[2] or one 64-bit integer)");
+	p.seed_dev = (const uint64_t*)seed.untyped_data();
 	return to_error(fa2_dropout_mask(&p, (uint8_t*)keep->untyped_data(), stream));
 }
 
@@ -144,13 +147,13 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(fa2_fwd_ffi, FwdImpl,
                                   .Arg<ffi::AnyBuffer>()  // v
                                   .Arg<ffi::AnyBuffer>()  // bias
                                   .Arg<ffi::AnyBuffer>()  // seqlens
+                                  .Arg<ffi::AnyBuffer>()  // seed
                                   .Ret<ffi::AnyBuffer>()  // o
                                   .Ret<ffi::AnyBuffer>()  // lse
                                   .Ret<ffi::AnyBuffer>()  // scratch
                                   .Attr<float>("scale")
                                   .Attr<float>("dropout_p")
                                   .Attr<bool>("causal")
-                                  .Attr<int64_t>("seed")
                                   .Attr<bool>("bias_group"));
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(fa2_bwd_ffi, BwdImpl,
@@ -161,6 +164,7 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(fa2_bwd_ffi, BwdImpl,
                                   .Arg<ffi::AnyBuffer>()  // v
                                   .Arg<ffi::AnyBuffer>()  // bias
                                   .Arg<ffi::AnyBuffer>()  // seqlens
+                                  .Arg<ffi::AnyBuffer>()  // seed
                                   .Arg<ffi::AnyBuffer>()  // o
                                   .Arg<ffi::AnyBuffer>()  // lse
                                   .Arg<ffi::AnyBuffer>()  // dout
@@ -171,12 +175,11 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(fa2_bwd_ffi, BwdImpl,
                                   .Attr<float>("scale")
                                   .Attr<float>("dropout_p")
                                   .Attr<bool>("causal")
-                                  .Attr<int64_t>("seed")
                                   .Attr<bool>("bias_group"));
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(fa2_dropout_mask_ffi, DropoutMaskImpl,
                               ffi::Ffi::Bind()
                                   .Ctx<ffi::PlatformStream<hipStream_t>>()
+                                  .Arg<ffi::AnyBuffer>()  // seed
                                   .Ret<ffi::AnyBuffer>()  // keep
-                                  .Attr<float>("dropout_p")
-                                  .Attr<int64_t>("seed"));
+                                  .Attr<float>("dropout_p"));

@@ -74,7 +74,7 @@ def _fill_common(p, q, k, v, bias, seqlens, scale, p_drop, causal, seed):
 	p.causal = 1 if causal else 0
 	p.scale = float(scale)
 	p.p_drop = float(p_drop)
-	p.seed = int(seed) & 0xFFFFFFFFFFFFFFFF
+	_fill_seed(p, seed, q.device)
 	p.q, p.k, p.v = _t4(q), _t4(k), _t4(v)
 	if bias is not None:
 		p.bias = bias.data_ptr()
@@ -88,6 +88,20 @@ def _fill_common(p, q, k, v, bias, seqlens, scale, p_drop, causal, seed):
 		p.bias_group = 1 if (bias.shape[1] == Hkv and Hkv != Hq and bias.shape[1] != 1) else 0
 	if seqlens is not None:
 		p.seqlens = seqlens.data_ptr()
+
+
+def _fill_seed(p, seed, device):
+	"""The dropout seed is a Python int (copied into the parameter block) or a one-element int64 tensor on the device,
+	which the kernels read there: a seed that is itself the result of device work - as a traced `dropout_seed` is in
+	the reference, an operand of the custom call (_forward_triton.py:553) - needs no host round trip."""
+	if isinstance(seed, torch.Tensor):
+		if seed.dtype != torch.int64 or seed.numel() != 1 or seed.device != device:
+			raise ValueError("a tensor dropout_seed must be a one-element int64 tensor on the device of q")
+		p.seed = 0
+		p.seed_dev = seed.data_ptr()
+	else:
+		p.seed = int(seed or 0) & 0xFFFFFFFFFFFFFFFF
+		p.seed_dev = None
 
 
 def _prep_bias(bias):
@@ -132,7 +146,7 @@ def fwd(q, k, v, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, 
 	out = torch.empty((B, Sq, Hq, D), dtype=q.dtype, device=q.device)
 	lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
 	p = _lib.new_params()
-	_fill_common(p, q, k, v, bias, seqlens, scale, dropout_prob, causal, dropout_seed or 0)
+	_fill_common(p, q, k, v, bias, seqlens, scale, dropout_prob, causal, dropout_seed)
 	p.o = _t4(out)
 	p.lse = lse.data_ptr()
 	# short query over many keys: scratch lets the library split the keys over workgroups
@@ -159,7 +173,7 @@ def bwd(q, k, v, out, lse, dout, bias=None, seqlens=None, softmax_scale=None, dr
 	dk = torch.empty_like(k, memory_format=torch.contiguous_format)
 	dv = torch.empty_like(v, memory_format=torch.contiguous_format)
 	p = _lib.new_params()
-	_fill_common(p, q, k, v, bias, seqlens, scale, dropout_prob, causal, dropout_seed or 0)
+	_fill_common(p, q, k, v, bias, seqlens, scale, dropout_prob, causal, dropout_seed)
 	p.o = _t4(out)
 	p.lse = lse.data_ptr()
 	p.dout, p.dq, p.dk, p.dv = _t4(dout), _t4(dq), _t4(dk), _t4(dv)
@@ -180,7 +194,7 @@ def dropout_mask(B, H, Sq, Sk, dropout_prob, dropout_seed, device) -> torch.Tens
 	p = _lib.new_params()
 	p.B, p.Hq, p.Hkv, p.Sq, p.Sk, p.D = B, H, H, Sq, Sk, 64
 	p.p_drop = float(dropout_prob)
-	p.seed = int(dropout_seed or 0) & 0xFFFFFFFFFFFFFFFF
+	_fill_seed(p, dropout_seed, torch.device(device))
 	_lib.check(lib.fa2_dropout_mask(ctypes.byref(p), keep.data_ptr(), _stream_ptr(device)))
 	return keep
 
@@ -201,7 +215,8 @@ class Plan:
 		self.out = torch.empty((B, Sq, Hq, D), dtype=q.dtype, device=q.device)
 		self.lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
 		p = self.params = _lib.new_params()
-		_fill_common(p, self.q, self.k, self.v, self.bias, seqlens, scale, dropout_prob, causal, dropout_seed or 0)
+		_fill_common(p, self.q, self.k, self.v, self.bias, seqlens, scale, dropout_prob, causal, dropout_seed)
+		self.seed = dropout_seed  # (a device-resident seed must outlive the plan's calls)
 		p.o = _t4(self.out)
 		p.lse = self.lse.data_ptr()
 		self.device = q.device

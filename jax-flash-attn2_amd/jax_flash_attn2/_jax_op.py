@@ -78,15 +78,32 @@ def _prep(q, k, v, bias, attention_mask):
 	return bias, seqlens, bias_group
 
 
-def _attrs(q, softmax_scale, dropout_prob, causal, dropout_seed, bias_group):
+def _attrs(q, softmax_scale, dropout_prob, causal, bias_group):
+	"""Attributes of the custom calls: compile-time constants only (the seed is an operand)."""
 	scale = 1.0 / math.sqrt(q.shape[-1]) if softmax_scale is None else softmax_scale
 	return dict(
 		scale=np.float32(scale),
 		dropout_p=np.float32(dropout_prob),
 		causal=bool(causal),
-		seed=np.int64(0 if dropout_seed is None else dropout_seed),
 		bias_group=bool(bias_group),
 	)
+
+
+def _seed_operand(dropout_seed):
+	"""The dropout seed as the 8-byte operand of the custom calls: uint32[2], low word first.
+	A Python int is split on the host; an array or tracer (the reference jits with a traced
+	dropout_seed, _flash_attention.py:91-92) is split with array operations, so nothing is
+	ever converted to a host scalar and one executable serves every seed."""
+	if dropout_seed is None:
+		return jnp.zeros((2,), jnp.uint32)
+	if isinstance(dropout_seed, (int, np.integer)):
+		s = int(dropout_seed) & 0xFFFFFFFFFFFFFFFF
+		return jnp.array([s & 0xFFFFFFFF, s >> 32], dtype=jnp.uint32)
+	x = jnp.asarray(dropout_seed).reshape(())
+	if x.dtype.itemsize == 8:
+		x = x.astype(jnp.uint64)
+		return jnp.stack([(x & 0xFFFFFFFF).astype(jnp.uint32), (x >> 32).astype(jnp.uint32)])
+	return jnp.stack([x.astype(jnp.uint32), jnp.zeros((), jnp.uint32)])
 
 
 def _fwd_scratch_bytes(q, k) -> int:
@@ -101,7 +118,7 @@ def _fwd_scratch_bytes(q, k) -> int:
 	return max(int(_lib.load().fa2_fwd_scratch_bytes(ctypes.byref(p))), 256)
 
 
-def _fwd_call(q, k, v, bias, seqlens, attrs):
+def _fwd_call(q, k, v, bias, seqlens, seed, attrs):
 	_register()
 	B, Sq, Hq, _ = q.shape
 	out_types = (
@@ -109,11 +126,11 @@ def _fwd_call(q, k, v, bias, seqlens, attrs):
 		jax.ShapeDtypeStruct((B, Hq, Sq), jnp.float32),
 		jax.ShapeDtypeStruct((_fwd_scratch_bytes(q, k),), jnp.uint8),
 	)
-	out, lse, _ = _ffi.ffi_call("fa2_fwd_ffi", out_types)(q, k, v, bias, seqlens, **attrs)
+	out, lse, _ = _ffi.ffi_call("fa2_fwd_ffi", out_types)(q, k, v, bias, seqlens, seed, **attrs)
 	return out, lse
 
 
-def _bwd_call(q, k, v, bias, seqlens, out, lse, dout, attrs):
+def _bwd_call(q, k, v, bias, seqlens, seed, out, lse, dout, attrs):
 	_register()
 	B, Sq, Hq, _ = q.shape
 	scratch_bytes = (B * Hq * Sq * 4 + 255) // 256 * 256  # fa2_bwd_scratch_bytes
@@ -123,10 +140,12 @@ def _bwd_call(q, k, v, bias, seqlens, out, lse, dout, attrs):
 		jax.ShapeDtypeStruct(v.shape, v.dtype),
 		jax.ShapeDtypeStruct((scratch_bytes,), jnp.uint8),
 	)
-	dq, dk, dv, _ = _ffi.ffi_call("fa2_bwd_ffi", out_types)(q, k, v, bias, seqlens, out, lse, dout, **attrs)
+	dq, dk, dv, _ = _ffi.ffi_call("fa2_bwd_ffi", out_types)(q, k, v, bias, seqlens, seed, out, lse, dout, **attrs)
 	return dq, dk, dv
 
 
+# static: softmax_scale, dropout_prob, causal, varlen_mode (as in the reference, _flash_attention.py:119); dropout_seed
+# (argument 8) is an ordinary operand and may be traced
 @functools.partial(jax.custom_vjp, nondiff_argnums=(5, 6, 7, 9))
 def flash_attention_call(q, k, v, attention_mask=None, bias=None, softmax_scale=None, dropout_prob=0.0, causal=False,
                          dropout_seed=None, varlen_mode=True):
@@ -135,16 +154,16 @@ def flash_attention_call(q, k, v, attention_mask=None, bias=None, softmax_scale=
 
 def _fwd_rule(q, k, v, attention_mask, bias, softmax_scale, dropout_prob, causal, dropout_seed, varlen_mode):
 	bias_op, seqlens, bias_group = _prep(q, k, v, bias, attention_mask)
-	attrs = _attrs(q, softmax_scale, dropout_prob, causal, dropout_seed, bias_group)
-	out, lse = _fwd_call(q, k, v, bias_op, seqlens, attrs)
+	attrs = _attrs(q, softmax_scale, dropout_prob, causal, bias_group)
+	out, lse = _fwd_call(q, k, v, bias_op, seqlens, _seed_operand(dropout_seed), attrs)
 	return out, (q, k, v, bias, attention_mask, out, lse, dropout_seed)
 
 
 def _bwd_rule(softmax_scale, dropout_prob, causal, varlen_mode, residual, dout):
 	q, k, v, bias, attention_mask, out, lse, dropout_seed = residual
 	bias_op, seqlens, bias_group = _prep(q, k, v, bias, attention_mask)
-	attrs = _attrs(q, softmax_scale, dropout_prob, causal, dropout_seed, bias_group)
-	dq, dk, dv = _bwd_call(q, k, v, bias_op, seqlens, out, lse, dout, attrs)
+	attrs = _attrs(q, softmax_scale, dropout_prob, causal, bias_group)
+	dq, dk, dv = _bwd_call(q, k, v, bias_op, seqlens, _seed_operand(dropout_seed), out, lse, dout, attrs)
 	return dq, dk, dv, None, None, None  # no gradient for mask, bias, seed (_flash_attention.py:88)
 
 
@@ -164,7 +183,7 @@ def flash_attention(
 	varlen_mode: bool = True,
 ):
 	"""Same signature as the reference's `triton_flash_attention` (_flash_attention.py:125-157).
-	`dropout_seed` must be a Python int here: it becomes an attribute of the custom call.
+	`dropout_seed` may be a Python int, an array or a tracer: it is an operand of the custom call.
 	A 4-D boolean mask becomes the bias where(mask, 0, finfo(dtype).min) (README.md:188)."""
 	if attention_mask is not None and attention_mask.ndim == 4:
 		assert bias is None, "Attention mask is not supported along with attention bias. Just use bias instead."
@@ -188,9 +207,7 @@ def flash_attention(
 def dropout_mask(B, H, Sq, Sk, dropout_prob, dropout_seed):
 	_register()
 	out_type = jax.ShapeDtypeStruct((B, H, Sq, Sk), jnp.uint8)
-	return _ffi.ffi_call("fa2_dropout_mask_ffi", out_type)(
-		dropout_p=np.float32(dropout_prob), seed=np.int64(0 if dropout_seed is None else dropout_seed)
-	)
+	return _ffi.ffi_call("fa2_dropout_mask_ffi", out_type)(_seed_operand(dropout_seed), dropout_p=np.float32(dropout_prob))
 
 
 def place_on_least_used_gpu(query, key, value, bias):

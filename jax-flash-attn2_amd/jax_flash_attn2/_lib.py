@@ -57,6 +57,7 @@ class Fa2Params(ctypes.Structure):
 		("dv", Fa2Tensor),
 		("scratch", ctypes.c_void_p),
 		("scratch_bytes", ctypes.c_uint64),
+		("seed_dev", ctypes.c_void_p),
 	]
 
 

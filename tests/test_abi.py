@@ -79,6 +79,24 @@ def test_validate_accepts_good_params():
 	assert _lib.load().fa2_bwd_scratch_bytes(ctypes.byref(p)) == 2 * 8 * 128 * 4
 
 
+def test_parameter_block_of_the_first_header_version_is_accepted():
+	"""struct_size of the block without the fields added later (seed_dev): the library fills them with zeros;
+	anything shorter is refused."""
+	P = _lib.Fa2Params
+	v1 = P.seed_dev.offset
+	p = _good_params()
+	p.seed_dev = 0xdead0008  # beyond struct_size: must not be looked at
+	p.struct_size = v1
+	assert _rc(p, 0) == 0 and _rc(p, 1) == 0
+	assert _lib.load().fa2_bwd_scratch_bytes(ctypes.byref(p)) == 2 * 8 * 128 * 4
+	p.struct_size = v1 - 8
+	assert _rc(p, 0) == -1
+	# a misaligned device seed pointer is refused
+	p = _good_params()
+	p.seed_dev = 0x60004
+	assert _rc(p, 0) == -5
+
+
 @pytest.mark.parametrize(
 	"mutate,code",
 	[

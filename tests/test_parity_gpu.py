@@ -295,6 +295,42 @@ def test_dropout_mask_is_bit_exact(B, H, Sq, Sk, p, seed):
 	assert np.array_equal(keep, O.dropout_keep_mask(seed, p, B, H, Sq, Sk))
 
 
+def test_seed_in_device_memory_gives_the_masks_of_the_host_seed():
+	"""The dropout seed as a run-time operand: a 64-bit value in device memory that the kernels read
+	(fa2_params.seed_dev) - as the reference hands dropout_seed to its custom call as an operand
+	(_forward_triton.py:553).  Forward, backward and the exported mask are bit-identical to the host-seed path."""
+	B, S, Hq, Hkv, D, p = 2, 200, 4, 2, 128, 0.2
+	q, k, v, do, _ = make_inputs(B, S, S, Hq, Hkv, D, torch.bfloat16, 5)
+	q, k, v, do = (_dev(t) for t in (q, k, v, do))
+	for seed in (42, (1 << 63) | 12345, 0):
+		signed = seed - (1 << 64) if seed >= (1 << 63) else seed
+		seed_t = torch.tensor([signed], dtype=torch.int64, device=DEV)
+		o0, lse0 = op.fwd(q, k, v, None, None, None, p, True, seed)
+		o1, lse1 = op.fwd(q, k, v, None, None, None, p, True, seed_t)
+		assert torch.equal(o0, o1) and torch.equal(lse0, lse1)
+		g0 = op.bwd(q, k, v, o0, lse0, do, None, None, None, p, True, seed)
+		g1 = op.bwd(q, k, v, o0, lse0, do, None, None, None, p, True, seed_t)
+		for a, b in zip(g0, g1):
+			assert torch.equal(a, b)
+		m0 = op.dropout_mask(B, Hq, S, S, p, seed, DEV)
+		m1 = op.dropout_mask(B, Hq, S, S, p, seed_t, DEV)
+		assert torch.equal(m0, m1)
+		assert np.array_equal(m1.cpu().numpy().astype(bool), O.dropout_keep_mask(seed, p, B, Hq, S, S))
+	# the seed is read at run time: a new value in the same buffer changes the mask of the next call
+	seed_t = torch.tensor([1], dtype=torch.int64, device=DEV)
+	m1 = op.dropout_mask(1, 1, 64, 64, 0.5, seed_t, DEV)
+	seed_t.fill_(2)
+	m2 = op.dropout_mask(1, 1, 64, 64, 0.5, seed_t, DEV)
+	assert np.array_equal(m2.cpu().numpy().astype(bool), O.dropout_keep_mask(2, 0.5, 1, 1, 64, 64)) and not torch.equal(m1, m2)
+	# the differentiation rule passes a device seed through as well
+	qq, kk, vv = (t.clone().requires_grad_() for t in (q, k, v))
+	out = op.flash_attention(qq, kk, vv, dropout_prob=p, causal=True, dropout_seed=torch.tensor([42], dtype=torch.int64, device=DEV))
+	out.backward(do)
+	o0, lse0 = op.fwd(q, k, v, None, None, None, p, True, 42)
+	g0 = op.bwd(q, k, v, o0, lse0, do, None, None, None, p, True, 42)
+	assert torch.equal(out.detach(), o0) and torch.equal(qq.grad, g0[0]) and torch.equal(kk.grad, g0[1])
+
+
 def test_kernels_apply_exactly_the_exported_mask():
 	"""Read the mask back out of each kernel: with q = 0 the probabilities are uniform,
 	and one-hot V / dO / K rows turn O, dV and dQ into scaled copies of the keep-mask."""
