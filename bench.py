@@ -99,6 +99,26 @@ def measured_traffic(workload, kernel):
 	return rec.get("hbm_bytes_per_launch") if rec.get("kernel") == kernel else None
 
 
+def mfma_peak(torch, dev):
+	"""What the chip sustains on bf16 matrix products alone (random operands), and at which clock."""
+	import ctypes
+
+	from jax_flash_attn2 import _lib
+
+	lib = _lib.load()
+	wgs, iters = 1024, 4000
+	buf = torch.zeros(16 + wgs * 1024, dtype=torch.uint8, device=dev)
+	st = torch.cuda.current_stream(dev).cuda_stream
+	run = lambda n: _lib.check(lib.fa2_bench_mfma(buf.data_ptr(), buf.numel(), wgs, n, st))
+	run(iters)  # settle the clocks
+	torch.cuda.synchronize()
+	ms = event_time_ms(lambda: run(iters), 3, torch)
+	ticks = buf[:16].cpu().view(torch.int64)
+	flops = wgs * 4.0 * iters * 32 * 32768
+	return {"tflops": flops / (ms * 1e-3) / 1e12, "clock_mhz": float(ticks[0]) / (float(ticks[1]) / 100.0),
+	        "what": "v_mfma_f32_32x32x16_bf16 only, random operands, 4 waves/CU x 4 independent chains"}
+
+
 def cpu_baseline(w):
 	"""Reference JAX-platform algorithm (NumPy restatement) on a bounded sample of the workload."""
 	sys.path.insert(0, os.path.join(ROOT, "oracle"))
@@ -117,23 +137,38 @@ def cpu_baseline(w):
 	k = rng.standard_normal((B, S, Hkv, D), dtype=np.float32) * 0.5
 	v = rng.standard_normal((B, S, Hkv, D), dtype=np.float32) * 0.5
 	do = rng.standard_normal((B, S, Hq, D), dtype=np.float32)
-	t0 = time.perf_counter()
-	if w["bwd"]:
-		O.jax_platform_call(q, k, v, with_grads_for=do)
-	else:
-		O.jax_platform_call(q, k, v)
-	dt = time.perf_counter() - t0
-	# that branch of the reference never applies the causal mask: it computes the full S x S problem
-	flops = 4.0 * B * Hq * S * S * D * (3.5 if w["bwd"] else 1.0)
-	return {
-		"value": flops / dt / 1e12,
+	def timed(mask):
+		t0 = time.perf_counter()
+		if w["bwd"]:
+			O.jax_platform_call(q, k, v, with_grads_for=do, mask=mask)
+		else:
+			O.jax_platform_call(q, k, v, mask=mask)
+		return time.perf_counter() - t0
+
+	cores = os.cpu_count() if not os.environ.get("OMP_NUM_THREADS") else int(os.environ["OMP_NUM_THREADS"])
+	mult = 3.5 if w["bwd"] else 1.0
+	what = f"B={B} Hq={Hq} Hkv={Hkv} S={S} D={D} fp32, {'fwd+bwd' if w['bwd'] else 'fwd'}, blocks 128x128"
+	# as the reference's facade runs it: that branch never applies the causal mask, it computes the full S x S problem
+	dt = timed(None)
+	out = {
+		"value": 4.0 * B * Hq * S * S * D * mult / dt / 1e12,
 		"unit": "TFLOP/s",
-		"cores": os.cpu_count() if not os.environ.get("OMP_NUM_THREADS") else int(os.environ["OMP_NUM_THREADS"]),
+		"cores": cores,
 		"kind": "port",
-		"sample": f"B={B} Hq={Hq} Hkv={Hkv} S={S} D={D} fp32 non-causal (the reference's JAX branch ignores causal), "
-		          f"{'fwd+bwd' if w['bwd'] else 'fwd'}, blocks 128x128, {dt:.1f} s",
+		"sample": f"{what}, non-causal (the reference's JAX branch ignores causal), {dt:.1f} s",
 		"seconds": dt,
 	}
+	if w["causal"]:
+		# the same functions given a causal mask (they then skip the blocks above the diagonal); FLOPs counted as for the GPU
+		tri = np.tril(np.ones((S, S), dtype=bool))[None, None]
+		dtc = timed(tri)
+		out["causal"] = {
+			"value": 2.0 * B * Hq * S * S * D * mult / dtc / 1e12,
+			"unit": "TFLOP/s",
+			"sample": f"{what}, causal mask with block skipping, {dtc:.1f} s",
+			"seconds": dtc,
+		}
+	return out
 
 
 def main():
@@ -143,6 +178,7 @@ def main():
 	ap.add_argument("--warmup", type=int, default=5)
 	ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
 	ap.add_argument("--no-cpu-baseline", action="store_true")
+	ap.add_argument("--no-mfma-peak", action="store_true", help="skip the matrix-product-only microbenchmark")
 	ap.add_argument("--copy-calibration", action="store_true",
 	                help="also run a plain 1 GiB device copy (known traffic) so that rocprofv3 FETCH_SIZE / WRITE_SIZE "
 	                     "readings of the attention kernels can be scaled")
@@ -199,14 +235,14 @@ def main():
 	total = ff * (3.5 if w["bwd"] else 1.0)
 	tflops = total / (ms * 1e-3) / 1e12
 
-	# per-kernel durations, HIP events on the launch stream
+	# per-kernel durations, HIP events on the launch stream.  The backward of a step is two launches: the dQ
+	# kernel, which also forms delta (stages 5), then the dK/dV kernel (stages 2); they are timed as launched there.
 	it = max(3, min(args.steps, 20))
 	kern = {"fwd": event_time_ms(plan.forward, it, torch)}
 	alg = {"fwd": ff}
 	if w["bwd"]:
-		kern["bwd_delta"] = event_time_ms(lambda: plan.backward(1), it, torch)
+		kern["bwd_dq"] = event_time_ms(lambda: plan.backward(5), it, torch)
 		kern["bwd_dkdv"] = event_time_ms(lambda: plan.backward(2), it, torch)
-		kern["bwd_dq"] = event_time_ms(lambda: plan.backward(4), it, torch)
 		# 5-product convention: S, dP, dV, dK belong to the dK/dV kernel (4 x 0.5 fwd), dQ to the dQ kernel;
 		# the dQ kernel's recomputation of S and dP is not counted.
 		alg["bwd_dkdv"] = 2.0 * ff
@@ -222,6 +258,7 @@ def main():
 		"unit": "TFLOP/s",
 		"frac": achieved / peak,
 		"traffic": measured_traffic(args.workload, dom),
+		"traffic_source": "committed rocprofv3 FETCH_SIZE / WRITE_SIZE runs (profiles/), not measured in this run",
 		"kernel_ms": {n: round(t, 4) for n, t in kern.items()},
 		"kernel_tflops": {n: round(alg[n] / (kern[n] * 1e-3) / 1e12, 1) for n in kern if n in alg},
 	}
@@ -243,6 +280,10 @@ def main():
 		"pct_of_mfma_peak": 100.0 * tflops / peak,
 		"roofline": roofline,
 	}
+	if not args.no_mfma_peak:
+		mp = mfma_peak(torch, dev)
+		out["mfma_peak_measured"] = mp
+		roofline["frac_of_measured_peak"] = achieved / mp["tflops"]
 	if not args.no_cpu_baseline:
 		out["cpu_baseline"] = cpu_baseline(w)
 	print(json.dumps(out))

@@ -135,10 +135,11 @@ int fa2_bwd(const fa2_params* p, void* hip_stream);
  * bit 0 = delta pre-pass (`_attn_bwd_preprocess`, _backward_triton.py:79-147),
  * bit 1 = dK/dV kernel (`_attn_bwd_block_dkdv`, :257-435),
  * bit 2 = dQ kernel (`_attn_bwd_block_dq`, :519-709).  fa2_bwd == stages 7.
- * With fewer than all three bits the dK/dV and dQ kernels read the delta an
- * earlier pre-pass left in scratch.  With all three the pre-pass is not
- * launched on its own: the dQ kernel forms delta from the O and dO rows it
- * holds, leaves it in scratch and runs before the dK/dV kernel. */
+ * Bits 0 and 2 together (5, 7): the pre-pass is not launched on its own; the dQ
+ * kernel forms delta from the O and dO rows it holds, leaves it in scratch and
+ * runs before the dK/dV kernel - so stages 5 followed by stages 2 are exactly
+ * the two launches of fa2_bwd.  Bit 0 alone launches the stand-alone pre-pass;
+ * bit 1 or bit 2 without bit 0 read the delta an earlier call left in scratch. */
 int fa2_bwd_stages(const fa2_params* p, void* hip_stream, int stages);
 
 /* Bytes of scratch fa2_bwd needs for these dimensions (0 on invalid params). */
@@ -167,6 +168,13 @@ int fa2_dropout_mask(const fa2_params* p, uint8_t* keep, void* hip_stream);
 /* Validate params exactly as fa2_fwd / fa2_bwd would, without launching
  * (host-only; usable without a GPU).  which: 0 = forward, 1 = backward. */
 int fa2_validate(const fa2_params* p, int which);
+
+/* Measurement aid (no counterpart in the reference): launches `workgroups` workgroups of 4 waves
+ * that each run `iters` x 32 v_mfma_f32_32x32x16_bf16 on random operands and nothing else.
+ * FLOPs = workgroups * 4 * iters * 32 * 32768; the caller times the launch.  scratch (device,
+ * >= 16 + workgroups * 1024 bytes): on completion its first two uint64 hold workgroup 0's
+ * shader-clock cycles and 100 MHz wall-clock ticks, i.e. the clock the chip sustained. */
+int fa2_bench_mfma(void* scratch, size_t scratch_bytes, int workgroups, int iters, void* hip_stream);
 
 const char* fa2_strerror(int code);
 int fa2_version(void);

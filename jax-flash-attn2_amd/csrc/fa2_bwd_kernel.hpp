@@ -1072,10 +1072,10 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 	int groups = a.B * a.Hkv;
 	a.xcd_remap = (groups % 8 == 0) ? 1 : 0;
 	if (BIAS && a.bias_sh == 0 && a.B % 8 == 0) a.xcd_remap = 2;
-	// All three stages requested: the dQ kernel forms delta itself and runs first, the dK/dV
-	// kernel reads the delta it left in scratch.  Otherwise (per-kernel timing) each stage
-	// is launched as asked and the dQ / dK/dV kernels read the delta of an earlier pre-pass.
-	const bool fused_delta = (a.stages & 7) == 7;
+	// Delta and dQ both requested (the whole backward, or stages 1 + 4): the dQ kernel forms delta
+	// itself and runs first, the dK/dV kernel reads the delta it left in scratch.  Otherwise each
+	// stage is launched as asked and the dQ / dK/dV kernels read the delta of an earlier pre-pass.
+	const bool fused_delta = (a.stages & 5) == 5;
 	a.dq_makes_delta = fused_delta ? 1 : 0;
 	if ((a.stages & 1) && !fused_delta) {
 		int64_t nrows = (int64_t)a.B * a.Sq * a.Hq;

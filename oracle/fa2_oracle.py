@@ -324,12 +324,15 @@ def blockwise_bwd(q, k, v, o, lse, dO, bias=None, mask=None, blocksize_q=128, bl
 
 
 def jax_platform_call(q, k, v, bias=None, softmax_scale=None, blocksize_q=128, blocksize_k=128,
-                      dtype=np.float32, with_grads_for=None):
+                      dtype=np.float32, with_grads_for=None, mask=None):
 	"""FlashAttention._compute_jax (flash_attention.py:324-349) followed by
 	flash_attention_jax/_flash_attention.py:98-133: repeat KV heads to Hq,
 	transpose to [B,H,S,D], clamp the block sizes to S, pre-scale q, run the
 	blockwise forward with mask=None.  causal / attention_mask / dropout never
 	reach the kernel on this branch of the reference.  q,k,v are [B,S,H,D].
+	`mask` (boolean [B|1,H|1,Sq,Sk], not what the facade passes) runs the same
+	functions the way their own `mask` argument does, causal block skip included
+	(flash_attention_jax/_flash_attention.py:98-133 with a mask).
 	With `with_grads_for=dO` also returns (dq, dk, dv) the way jax.grad would
 	(chain rule through the repeat and the pre-scale)."""
 	B, Sq, Hq, D = q.shape
@@ -345,12 +348,12 @@ def jax_platform_call(q, k, v, bias=None, softmax_scale=None, blocksize_q=128, b
 	bb = None
 	if bias is not None:
 		bb = _expand_bias(bias, B, Hq, Hkv, Sq, kt.shape[2], dtype)
-	o, lse = blockwise_fwd(qt, kt, vt, bb, None, bq, bk, dtype)
+	o, lse = blockwise_fwd(qt, kt, vt, bb, mask, bq, bk, dtype)
 	out = np.swapaxes(o, 1, 2)
 	if with_grads_for is None:
 		return out
 	dOt = np.ascontiguousarray(np.swapaxes(with_grads_for, 1, 2)).astype(dtype)
-	dq, dk, dv = blockwise_bwd(qt, kt, vt, o, lse, dOt, bb, None, bq, bk)
+	dq, dk, dv = blockwise_bwd(qt, kt, vt, o, lse, dOt, bb, mask, bq, bk)
 	dq = np.swapaxes(dq, 1, 2) * dtype(sc)
 	dk = np.swapaxes(dk, 1, 2).reshape(B, -1, Hkv, r, D).sum(3)
 	dv = np.swapaxes(dv, 1, 2).reshape(B, -1, Hkv, r, D).sum(3)

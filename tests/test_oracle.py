@@ -192,6 +192,11 @@ def test_blockwise_restatement_equals_closed_form():
 	ob, lse = O.blockwise_fwd(qt / 4.0, kt, vt, mask=tri, dtype=np.float64, blocksize_q=64, blocksize_k=64)
 	oc, _ = O.attention_fwd(q, k, v, causal=True)
 	assert np.abs(np.swapaxes(ob, 1, 2) - oc).max() < 1e-6
+	# ... and so does the backward (the causal leg of the CPU baseline runs exactly this)
+	oc2, gc = O.jax_platform_call(q, k, v, dtype=np.float64, with_grads_for=dO, mask=tri, blocksize_q=64, blocksize_k=64)
+	assert np.abs(oc2 - oc).max() < 1e-6
+	for a, b in zip(gc, O.attention_bwd(q, k, v, dO, causal=True)):
+		assert np.abs(a - b).max() < 1e-5
 
 
 def test_bf16_helpers_round_trip():
