@@ -35,6 +35,9 @@ WORKLOADS = {
 	           desc="Llama-3-8B prefill B4 S4096 Hq32 Hkv8 D128 bf16 causal, forward+backward"),
 	"c3": dict(B=8, S=2048, Hq=16, Hkv=16, D=64, dtype="bf16", causal=False, bias=True, p=0.0, bwd=True,
 	           desc="padded MHA B8 S2048 H16 D64 bf16, bias [B,1,S,S] with mask folded in, forward+backward"),
+	"c3_split": dict(B=8, S=2048, Hq=16, Hkv=16, D=64, dtype="bf16", causal=False, bias=True, p=0.0, bwd=True, split_mask=True,
+	                 desc="padded MHA B8 S2048 H16 D64 bf16, bias [B,1,S,S] and the per-row key lengths passed separately "
+	                      "(kv_lens), forward+backward"),
 	"c4": dict(B=1, S=32768, Hq=64, Hkv=8, D=128, dtype="bf16", causal=True, bias=False, p=0.0, bwd=True,
 	           desc="long context B1 S32768 Hq64 Hkv8 D128 bf16 causal, forward+backward"),
 	"c5": dict(B=8, S=2048, Hq=16, Hkv=16, D=256, dtype="bf16", causal=True, bias=False, p=0.1, bwd=True,
@@ -63,7 +66,7 @@ def make_inputs(w, device):
 	k = rnd(1, (B, S, Hkv, D), mul)
 	v = rnd(2, (B, S, Hkv, D), mul)
 	do = rnd(3, (B, S, Hq, D), 1.0)
-	bias = None
+	bias = kv_lens = None
 	if w["bias"]:
 		# bias[b,0,i,j] = 1/(1+|i-j|) ; keys beyond a per-row valid length get finfo.min
 		i = torch.arange(S, device=device)
@@ -72,8 +75,12 @@ def make_inputs(w, device):
 		lens = torch.randint(S // 2, S + 1, (B,), generator=g, device=device)
 		valid = i[None, :] < lens[:, None]
 		bias = base[None, None].expand(B, 1, S, S).clone()
-		bias = torch.where(valid[:, None, None, :], bias, torch.full_like(bias, torch.finfo(dt).min)).to(dt)
-	return q, k, v, do, bias
+		if w.get("split_mask"):
+			bias = bias.to(dt)
+			kv_lens = lens.to(torch.int32).contiguous()
+		else:
+			bias = torch.where(valid[:, None, None, :], bias, torch.full_like(bias, torch.finfo(dt).min)).to(dt)
+	return q, k, v, do, bias, kv_lens
 
 
 def event_time_ms(fn, iters, torch):
@@ -197,9 +204,9 @@ def main():
 		sys.exit(1)
 	dev = torch.device("cuda:0")
 	w = WORKLOADS[args.workload]
-	q, k, v, do, bias = make_inputs(w, dev)
+	q, k, v, do, bias, kv_lens = make_inputs(w, dev)
 	plan = op.Plan(q, k, v, dout=do if w["bwd"] else None, bias=bias, causal=w["causal"], dropout_prob=w["p"],
-	               dropout_seed=42 if w["p"] > 0 else None)
+	               dropout_seed=42 if w["p"] > 0 else None, kv_lens=kv_lens)
 
 	def step():
 		plan.forward()
@@ -232,6 +239,9 @@ def main():
 	ms = (time.perf_counter() - t0) * 1e3 / args.steps
 
 	ff = fwd_flops(w)
+	if kv_lens is not None:
+		# only the valid keys count as work
+		ff *= float(kv_lens.float().mean()) / w["S"]
 	total = ff * (3.5 if w["bwd"] else 1.0)
 	tflops = total / (ms * 1e-3) / 1e12
 

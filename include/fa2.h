@@ -30,7 +30,7 @@ extern "C" {
 
 /* Element types; the values mirror dtype_index() in
  * jax_flash_attn2/flash_attention_triton/_utils.py:75-82. */
-enum { FA2_FP16 = 1, FA2_BF16 = 2, FA2_FP32 = 3 /* bias only */ };
+enum { FA2_FP16 = 1, FA2_BF16 = 2, FA2_FP32 = 3 /* bias only */, FA2_MASK_U8 = 4 /* bias only: boolean mask, see `bias` */ };
 
 /* Return codes. 0 = success, negative = error; nothing is launched on error. */
 enum {
@@ -82,7 +82,12 @@ typedef struct fa2_params {
 	 * bias_group != 0: the head axis has Hkv entries and q-head h reads entry
 	 * h / (Hq/Hkv) (flash_attention.py:161-164 materialises this repeat).   */
 	const void* bias;       /* NULL = no bias                              */
-	int32_t bias_dtype;     /* FA2_FP16 | FA2_BF16 | FA2_FP32              */
+	int32_t bias_dtype;     /* FA2_FP16 | FA2_BF16 | FA2_FP32, or FA2_MASK_U8: `bias` then points to a
+	                           boolean mask, one byte per position (0 = masked), same shape and stride
+	                           rules with strides in bytes.  A masked position adds the lowest finite
+	                           value of `dtype` to the score - exactly what the bias
+	                           where(mask, 0, finfo(dtype).min) of README.md:188 does, at one byte
+	                           per position instead of two or four */
 	int32_t bias_group;
 	int64_t bias_stride_b, bias_stride_h, bias_stride_m;
 
@@ -110,6 +115,13 @@ typedef struct fa2_params {
 	 * (_forward_triton.py:553, _flash_attention.py:91-92) - and changing it needs neither a
 	 * new parameter block nor, under XLA, a new executable.                              */
 	const uint64_t* seed_dev;
+
+	/* Optional per-batch number of valid KEYS: keys j >= kv_lens[b] are masked, query rows
+	 * are not touched and causal stays aligned to the full Sk.  Unlike `seqlens` it may be
+	 * combined with a bias and with Sq != Sk (key padding of cross attention, or of a
+	 * batch that also carries a bias); key tiles beyond the length are skipped, not
+	 * masked.  A row left without any allowed key gives O = 0 and lse = -inf.       */
+	const int32_t* kv_lens; /* [B] int32 on device, NULL = all Sk keys     */
 } fa2_params;
 
 /* sizeof(fa2_params) in the first version of this header: up to and including scratch_bytes */

@@ -41,7 +41,7 @@ int check_tensor(const fa2_tensor& t, bool required) {
 	return FA2_OK;
 }
 
-int esize(int dtype) { return dtype == FA2_FP32 ? 4 : 2; }
+int esize(int dtype) { return dtype == FA2_FP32 ? 4 : dtype == FA2_MASK_U8 ? 1 : 2; }
 
 KTensor conv(const fa2_tensor& t) {
 	KTensor k;
@@ -69,7 +69,8 @@ int validate(const fa2_params* p, int which, bool own_scratch = false) {
 	if ((rc = check_tensor(p->o, true))) return rc;
 	if (!p->lse || ((uintptr_t)p->lse & 3)) return FA2_EINVAL_PTR;
 	if (p->bias) {
-		if (p->bias_dtype != FA2_FP16 && p->bias_dtype != FA2_BF16 && p->bias_dtype != FA2_FP32) return FA2_EINVAL_BIAS;
+		if (p->bias_dtype != FA2_FP16 && p->bias_dtype != FA2_BF16 && p->bias_dtype != FA2_FP32 && p->bias_dtype != FA2_MASK_U8)
+			return FA2_EINVAL_BIAS;
 		if (((uintptr_t)p->bias % esize(p->bias_dtype)) != 0) return FA2_EINVAL_BIAS;
 		if (p->bias_stride_b < 0 || p->bias_stride_h < 0 || p->bias_stride_m < p->Sk) return FA2_EINVAL_BIAS;
 	}
@@ -77,6 +78,7 @@ int validate(const fa2_params* p, int which, bool own_scratch = false) {
 		if (p->bias || p->Sq != p->Sk) return FA2_EINVAL_MASK;
 		if ((uintptr_t)p->seqlens & 3) return FA2_EINVAL_PTR;
 	}
+	if (p->kv_lens && ((uintptr_t)p->kv_lens & 3)) return FA2_EINVAL_PTR;
 	if (which == 1) {
 		if ((rc = check_tensor(p->dout, true))) return rc;
 		if ((rc = check_tensor(p->dq, true))) return rc;
@@ -112,7 +114,10 @@ void fill(const fa2_params* p, KArgs& a) {
 		a.bias_sm = p->bias_stride_m * es;
 		a.bias_dtype = p->bias_dtype;
 		a.bias_group = p->bias_group ? 1 : 0;
-		int valign = es == 4 ? 16 : 8;
+		int valign = es == 4 ? 16 : es == 2 ? 8 : 4;
+		// a masked position of a boolean mask adds the lowest finite value of the element type, which is what
+		// where(mask, 0, finfo(dtype).min) passed as a bias would add
+		a.mask_fill = p->dtype == FA2_BF16 ? -3.38953139e38f : -65504.f;
 		a.bias_vec4 = (((uintptr_t)p->bias % valign) == 0 && a.bias_sb % valign == 0 && a.bias_sh % valign == 0 &&
 		               a.bias_sm % valign == 0)
 		                  ? 1
@@ -125,6 +130,7 @@ void fill(const fa2_params* p, KArgs& a) {
 		                 : 0;
 	}
 	a.seqlens = p->seqlens;
+	a.kv_lens = p->kv_lens;
 	a.B = p->B;
 	a.Sq = p->Sq;
 	a.Sk = p->Sk;

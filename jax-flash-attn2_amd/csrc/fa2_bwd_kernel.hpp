@@ -136,6 +136,11 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		sk_eff = len;
 	}
 	const int off = sk_eff - sq_eff;
+	if (a.kv_lens) {  // key padding only: the causal alignment keeps counting from the full key count
+		int len = a.kv_lens[b];
+		len = len < 0 ? 0 : len;
+		sk_eff = len < sk_eff ? len : sk_eff;
+	}
 	const int n0 = nt * BN;
 	const int wn0 = n0 + 32 * w;
 	const int jcol = wn0 + c;  // this lane's key
@@ -261,7 +266,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		if constexpr (BIAS) {
 			int hb = a.bias_group ? hk : hq;
 			int jc = jcol < a.Sk ? jcol : a.Sk - 1;
-			int es = a.bias_dtype == 3 ? 4 : 2;
+			int es = a.bias_dtype == 3 ? 4 : a.bias_dtype == 4 ? 1 : 2;
 			bias_base = a.bias + (int64_t)b * a.bias_sb + (int64_t)hb * a.bias_sh + (int64_t)jc * es;
 		}
 		// The tile's QB blocks of 32 rows go through three stages,
@@ -322,9 +327,10 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 				if constexpr (BIAS_T)
 					bv[qb & 1][i] = (float)*(const typename T::E*)pp;
 				else
-					bv[qb & 1][i] = a.bias_dtype == 3 ? *(const float*)pp
+					bv[qb & 1][i] = a.bias_dtype == 3   ? *(const float*)pp
 					                : a.bias_dtype == 2 ? (float)*(const __bf16*)pp
-					                                    : (float)*(const _Float16*)pp;
+					                : a.bias_dtype == 1 ? (float)*(const _Float16*)pp
+					                                    : (*(const uint8_t*)pp ? 0.f : a.mask_fill);
 			}
 		};
 		// bias values of block qb that belong to slot j when the 16 of them are spread over a stage
@@ -747,6 +753,11 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 		sk_eff = len;
 	}
 	const int off = sk_eff - sq_eff;
+	if (a.kv_lens) {  // key padding only: the causal alignment keeps counting from the full key count
+		int len = a.kv_lens[b];
+		len = len < 0 ? 0 : len;
+		sk_eff = len < sk_eff ? len : sk_eff;
+	}
 	const int m0 = mt * BM;
 	const int wm0 = m0 + w * (QB * 32);
 
@@ -911,7 +922,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 					const char* rowp = bias_base + (int64_t)i * a.bias_sm;
 #pragma unroll
 					for (int aa = 0; aa < 4; ++aa)
-						bv[qb][aa] = load_bias4(rowp, n0 + 32 * kb + 8 * aa + 4 * g, a.bias_dtype, a.bias_vec4, a.Sk);
+						bv[qb][aa] = load_bias4(rowp, n0 + 32 * kb + 8 * aa + 4 * g, a.bias_dtype, a.bias_vec4, a.Sk, a.mask_fill);
 				}
 			}
 			f32x16 s[QB], dp[QB];

@@ -63,8 +63,9 @@ FA2_DEV void decode_block(const KArgs& a, int& mt, int& h, int& b, int id = (int
 	h = hk * r + within % r;
 }
 
-// four consecutive bias values bias[row][col..col+3] as floats
-FA2_DEV f32x4 load_bias4(const char* rowp, int col, int dtype, bool vec_ok, int ncols) {
+// four consecutive bias values bias[row][col..col+3] as floats.  dtype 4: the row holds bytes of a boolean
+// mask; a zero byte stands for the additive value `fill`, anything else for 0.
+FA2_DEV f32x4 load_bias4(const char* rowp, int col, int dtype, bool vec_ok, int ncols, float fill) {
 	f32x4 out;
 	if (vec_ok && col + 3 < ncols) {
 		if (dtype == 3) {
@@ -72,9 +73,13 @@ FA2_DEV f32x4 load_bias4(const char* rowp, int col, int dtype, bool vec_ok, int 
 		} else if (dtype == 2) {
 			bf16x4 t = *(const bf16x4*)(rowp + (int64_t)col * 2);
 			out = __builtin_convertvector(t, f32x4);
-		} else {
+		} else if (dtype == 1) {
 			f16x4 t = *(const f16x4*)(rowp + (int64_t)col * 2);
 			out = __builtin_convertvector(t, f32x4);
+		} else {
+			uint32_t t = *(const uint32_t*)(rowp + col);
+#pragma unroll
+			for (int e = 0; e < 4; ++e) out[e] = ((t >> (8 * e)) & 0xffu) ? 0.f : fill;
 		}
 	} else {
 #pragma unroll
@@ -85,8 +90,10 @@ FA2_DEV f32x4 load_bias4(const char* rowp, int col, int dtype, bool vec_ok, int 
 					x = *(const float*)(rowp + (int64_t)(col + e) * 4);
 				else if (dtype == 2)
 					x = (float)*(const __bf16*)(rowp + (int64_t)(col + e) * 2);
-				else
+				else if (dtype == 1)
 					x = (float)*(const _Float16*)(rowp + (int64_t)(col + e) * 2);
+				else
+					x = *(const uint8_t*)(rowp + col + e) ? 0.f : fill;
 			}
 			out[e] = x;
 		}
@@ -160,6 +167,11 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 		sk_eff = len;
 	}
 	const int off = sk_eff - sq_eff;  // causal: key j allowed for row i iff j <= i + off
+	if (a.kv_lens) {  // key padding only: the causal alignment keeps counting from the full key count
+		int len = a.kv_lens[b];
+		len = len < 0 ? 0 : len;
+		sk_eff = len < sk_eff ? len : sk_eff;
+	}
 	const int m0 = mt * BM;
 	const int wm0 = m0 + w * (QB * 32);
 
@@ -346,7 +358,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 				for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
 					for (int aa = 0; aa < 4; ++aa)
-						bv[kb][qb][aa] = load_bias4(rowp, n0 + 32 * kb + 8 * aa + 4 * g, a.bias_dtype, a.bias_vec4, a.Sk);
+						bv[kb][qb][aa] = load_bias4(rowp, n0 + 32 * kb + 8 * aa + 4 * g, a.bias_dtype, a.bias_vec4, a.Sk, a.mask_fill);
 			}
 		}
 

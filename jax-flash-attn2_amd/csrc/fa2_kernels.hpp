@@ -18,11 +18,13 @@ struct KArgs {
 	float* delta;    // [B, Hq, Sq] rowsum(dO * O)  (backward scratch)
 	const char* bias;
 	int64_t bias_sb, bias_sh, bias_sm;  // bytes
-	int bias_dtype;  // FA2_FP16 / FA2_BF16 / FA2_FP32
+	int bias_dtype;  // FA2_FP16 / FA2_BF16 / FA2_FP32 / FA2_MASK_U8 (bytes: 0 = masked, taken as the bias mask_fill)
 	int bias_group;  // head axis of bias indexed by kv-head
 	int bias_vec4;   // rows are 4-element aligned: vector loads allowed
+	float mask_fill; // FA2_MASK_U8: the additive value of a masked position = lowest finite value of the element type
 	int bias_lds;    // bias tiles may be copied global->LDS in 16-byte pieces (see fa2_api.hip)
 	const int32_t* seqlens;
+	const int32_t* kv_lens;  // [B]: keys at or beyond kv_lens[b] are masked (query rows unaffected)
 	int B, Sq, Sk, Hq, Hkv;
 	int causal;
 	float scale;

@@ -23,10 +23,11 @@ import torch
 
 from . import _lib
 from ._checks import check_shapes  # noqa: F401  (re-exported)
-from ._lib import FA2_BF16, FA2_FP16, FA2_FP32, Fa2Tensor
+from ._lib import FA2_BF16, FA2_FP16, FA2_FP32, FA2_MASK_U8, Fa2Tensor
 
 _DTYPES = {torch.float16: FA2_FP16, torch.bfloat16: FA2_BF16}
-_BIAS_DTYPES = {torch.float16: FA2_FP16, torch.bfloat16: FA2_BF16, torch.float32: FA2_FP32}
+# (a uint8 / bool `bias` is a boolean mask, one byte per position: see fa2_params.bias_dtype)
+_BIAS_DTYPES = {torch.float16: FA2_FP16, torch.bfloat16: FA2_BF16, torch.float32: FA2_FP32, torch.uint8: FA2_MASK_U8}
 
 
 def _stream_ptr(device) -> int:
@@ -66,7 +67,7 @@ def _usable(x: torch.Tensor) -> torch.Tensor:
 	return x
 
 
-def _fill_common(p, q, k, v, bias, seqlens, scale, p_drop, causal, seed):
+def _fill_common(p, q, k, v, bias, seqlens, scale, p_drop, causal, seed, kv_lens=None):
 	B, Sq, Hq, D = q.shape
 	Sk, Hkv = k.shape[1], k.shape[2]
 	p.dtype = _DTYPES[q.dtype]
@@ -88,6 +89,10 @@ def _fill_common(p, q, k, v, bias, seqlens, scale, p_drop, causal, seed):
 		p.bias_group = 1 if (bias.shape[1] == Hkv and Hkv != Hq and bias.shape[1] != 1) else 0
 	if seqlens is not None:
 		p.seqlens = seqlens.data_ptr()
+	if kv_lens is not None:
+		if kv_lens.dtype != torch.int32 or kv_lens.numel() != B or not kv_lens.is_contiguous():
+			raise ValueError("kv_lens must be a contiguous int32 tensor with one entry per batch row")
+		p.kv_lens = kv_lens.data_ptr()
 
 
 def _fill_seed(p, seed, device):
@@ -107,6 +112,8 @@ def _fill_seed(p, seed, device):
 def _prep_bias(bias):
 	if bias is None:
 		return None
+	if bias.dtype == torch.bool:
+		bias = bias.view(torch.uint8)  # same bytes: 0 = masked
 	if bias.dtype not in _BIAS_DTYPES:
 		bias = bias.to(torch.float32)
 	if bias.stride(3) != 1:
@@ -114,13 +121,14 @@ def _prep_bias(bias):
 	return bias
 
 
-def _mask_to_bias(mask, q):
-	"""A 4-D boolean mask [B|1, H|1, Sq, Sk] as the additive bias where(mask, 0, finfo(dtype).min) - the recipe the
-	reference's documentation gives for general masks (README.md:188).  Its GPU path itself only takes the 2-D mask."""
+def _mask_operand(mask, q):
+	"""A 4-D boolean mask [B|1, H|1, Sq, Sk] is handed to the kernels as it is, one byte per position.  They add the
+	lowest finite value of q's dtype at masked positions, i.e. they compute what the reference's documentation
+	spells as the bias where(mask, 0, finfo(dtype).min) (README.md:188) without that bias ever being built.
+	(The reference's GPU path itself only takes the 2-D mask.)"""
 	m = mask.to(device=q.device)
 	m = m if m.dtype == torch.bool else m.ne(0)
-	zero = torch.zeros((), dtype=q.dtype, device=q.device)
-	return torch.where(m, zero, torch.full((), torch.finfo(q.dtype).min, dtype=q.dtype, device=q.device))
+	return m.contiguous() if m.stride(3) != 1 else m
 
 
 def _seqlens_from_mask(attention_mask, q):
@@ -134,7 +142,7 @@ def _seqlens_from_mask(attention_mask, q):
 	return attention_mask.to(device=q.device).ne(0).sum(dim=1, dtype=torch.int32).contiguous()
 
 
-def fwd(q, k, v, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, causal=False, dropout_seed=None):
+def fwd(q, k, v, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, causal=False, dropout_seed=None, kv_lens=None):
 	"""Returns (out [B,Sq,Hq,D] in q.dtype, lse [B,Hq,Sq] fp32 natural log)."""
 	lib = _lib.load()
 	D0 = q.shape[-1]
@@ -146,7 +154,7 @@ def fwd(q, k, v, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, 
 	out = torch.empty((B, Sq, Hq, D), dtype=q.dtype, device=q.device)
 	lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
 	p = _lib.new_params()
-	_fill_common(p, q, k, v, bias, seqlens, scale, dropout_prob, causal, dropout_seed)
+	_fill_common(p, q, k, v, bias, seqlens, scale, dropout_prob, causal, dropout_seed, kv_lens)
 	p.o = _t4(out)
 	p.lse = lse.data_ptr()
 	# short query over many keys: scratch lets the library split the keys over workgroups
@@ -160,7 +168,7 @@ def fwd(q, k, v, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, 
 
 
 def bwd(q, k, v, out, lse, dout, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, causal=False,
-        dropout_seed=None):
+        dropout_seed=None, kv_lens=None):
 	"""Returns (dq, dk, dv) in the dtypes of q, k, v; dk/dv summed over each KV group."""
 	lib = _lib.load()
 	D0 = q.shape[-1]
@@ -173,7 +181,7 @@ def bwd(q, k, v, out, lse, dout, bias=None, seqlens=None, softmax_scale=None, dr
 	dk = torch.empty_like(k, memory_format=torch.contiguous_format)
 	dv = torch.empty_like(v, memory_format=torch.contiguous_format)
 	p = _lib.new_params()
-	_fill_common(p, q, k, v, bias, seqlens, scale, dropout_prob, causal, dropout_seed)
+	_fill_common(p, q, k, v, bias, seqlens, scale, dropout_prob, causal, dropout_seed, kv_lens)
 	p.o = _t4(out)
 	p.lse = lse.data_ptr()
 	p.dout, p.dq, p.dk, p.dv = _t4(dout), _t4(dq), _t4(dk), _t4(dv)
@@ -205,7 +213,7 @@ class Plan:
 	enqueue kernels, nothing is allocated per call."""
 
 	def __init__(self, q, k, v, dout=None, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, causal=False,
-	             dropout_seed=None):
+	             dropout_seed=None, kv_lens=None):
 		self.lib = _lib.load()
 		self.q, self.k, self.v = _usable(q), _usable(k), _usable(v)
 		self.bias = _prep_bias(bias)
@@ -215,7 +223,8 @@ class Plan:
 		self.out = torch.empty((B, Sq, Hq, D), dtype=q.dtype, device=q.device)
 		self.lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
 		p = self.params = _lib.new_params()
-		_fill_common(p, self.q, self.k, self.v, self.bias, seqlens, scale, dropout_prob, causal, dropout_seed)
+		self.kv_lens = kv_lens
+		_fill_common(p, self.q, self.k, self.v, self.bias, seqlens, scale, dropout_prob, causal, dropout_seed, kv_lens)
 		self.seed = dropout_seed  # (a device-resident seed must outlive the plan's calls)
 		p.o = _t4(self.out)
 		p.lse = self.lse.data_ptr()
@@ -252,18 +261,18 @@ class _FlashAttentionFn(torch.autograd.Function):
 	(_flash_attention.py:119-122).  Returns (dq, dk, dv) and None for everything else."""
 
 	@staticmethod
-	def forward(ctx, q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed):
-		out, lse = fwd(q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed)
-		ctx.save_for_backward(q, k, v, bias, seqlens, out, lse)
+	def forward(ctx, q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens=None):
+		out, lse = fwd(q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens)
+		ctx.save_for_backward(q, k, v, bias, seqlens, out, lse, kv_lens)
 		ctx.cfg = (softmax_scale, dropout_prob, causal, dropout_seed)
 		return out
 
 	@staticmethod
 	def backward(ctx, dout):
-		q, k, v, bias, seqlens, out, lse = ctx.saved_tensors
+		q, k, v, bias, seqlens, out, lse, kv_lens = ctx.saved_tensors
 		softmax_scale, dropout_prob, causal, dropout_seed = ctx.cfg
-		dq, dk, dv = bwd(q, k, v, out, lse, dout, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed)
-		return dq, dk, dv, None, None, None, None, None, None
+		dq, dk, dv = bwd(q, k, v, out, lse, dout, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens)
+		return dq, dk, dv, None, None, None, None, None, None, None
 
 
 def flash_attention(
@@ -277,15 +286,19 @@ def flash_attention(
 	causal: bool = False,
 	dropout_seed: tp.Optional[int] = None,
 	varlen_mode: bool = True,
+	*,
+	kv_lens=None,
 ):
 	"""Same signature as the reference's `triton_flash_attention`
 	(_flash_attention.py:125-157).  `varlen_mode` is accepted for source
 	compatibility; padded batches are always handled in-kernel from per-row
-	lengths, never by packing."""
+	lengths, never by packing.  `kv_lens` (keyword only, not in the reference):
+	int32 [B] number of valid keys per batch row - key padding that may be combined
+	with a bias and with Sq != Sk, which the 2-D attention_mask may not."""
 	del varlen_mode
 	if attention_mask is not None and attention_mask.dim() == 4:
 		assert bias is None, "Attention mask is not supported along with attention bias. Just use bias instead."
-		bias, attention_mask = _mask_to_bias(attention_mask, q), None
+		bias, attention_mask = _mask_operand(attention_mask, q), None
 	check_shapes(q, k, v, bias, attention_mask)
 	seqlens = _seqlens_from_mask(attention_mask, q)
-	return _FlashAttentionFn.apply(q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed)
+	return _FlashAttentionFn.apply(q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens)

@@ -10,7 +10,7 @@ import ctypes
 import os
 import threading
 
-FA2_FP16, FA2_BF16, FA2_FP32 = 1, 2, 3
+FA2_FP16, FA2_BF16, FA2_FP32, FA2_MASK_U8 = 1, 2, 3, 4
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(os.path.dirname(_HERE), "libfa2_hip.so")
@@ -58,6 +58,7 @@ class Fa2Params(ctypes.Structure):
 		("scratch", ctypes.c_void_p),
 		("scratch_bytes", ctypes.c_uint64),
 		("seed_dev", ctypes.c_void_p),
+		("kv_lens", ctypes.c_void_p),
 	]
 
 

@@ -127,13 +127,15 @@ def _expand_bias(bias, B, Hq, Hkv, Sq, Sk, dtype):
 	return np.broadcast_to(bias, (B, Hq, Sq, Sk))
 
 
-def allowed_mask(B, Sq, Sk, causal, seqlens=None):
+def allowed_mask(B, Sq, Sk, causal, seqlens=None, kv_lens=None):
 	"""allowed[b,i,j]: causal is bottom-right aligned (j <= i + Sk - Sq),
 	_forward_triton.py:127-132, refrence_call.py:66-67.  `seqlens[b]` is the
 	right-padded 2-D validity mask of the reference's GPU path reduced to a
 	length: keys j >= len are masked and query rows i >= len produce zeros
 	(_forward_triton.py:474-481,499-510,590-591).  With seqlens the causal
-	offset is 0 (it requires Sq == Sk)."""
+	offset is 0 (it requires Sq == Sk).  `kv_lens[b]` (not in the reference:
+	plain key padding) masks keys j >= len only; rows and the causal offset
+	are untouched."""
 	i = np.arange(Sq)[:, None]
 	j = np.arange(Sk)[None, :]
 	ok = np.ones((B, Sq, Sk), dtype=bool)
@@ -142,6 +144,8 @@ def allowed_mask(B, Sq, Sk, causal, seqlens=None):
 	if seqlens is not None:
 		L = np.asarray(seqlens).reshape(B, 1, 1)
 		ok &= (j[None] < L) & (i[None] < L)
+	if kv_lens is not None:
+		ok &= j[None] < np.asarray(kv_lens).reshape(B, 1, 1)
 	return ok
 
 
@@ -165,7 +169,7 @@ def _ptx(p, x):
 	return np.swapaxes(np.matmul(np.swapaxes(p, 2, 3), _bh(x)), 1, 2)
 
 
-def _scores(q, k, bias, scale, causal, seqlens, dtype):
+def _scores(q, k, bias, scale, causal, seqlens, dtype, kv_lens=None):
 	B, Sq, Hq, D = q.shape
 	_, Sk, Hkv, _ = k.shape
 	if Hq % Hkv:
@@ -177,13 +181,13 @@ def _scores(q, k, bias, scale, causal, seqlens, dtype):
 	bb = _expand_bias(bias, B, Hq, Hkv, Sq, Sk, dtype)
 	if bb is not None:
 		s = s + bb
-	ok = allowed_mask(B, Sq, Sk, causal, seqlens)[:, None]
+	ok = allowed_mask(B, Sq, Sk, causal, seqlens, kv_lens)[:, None]
 	s = np.where(ok, s, -np.inf)
 	return s, ok, r
 
 
 def attention_fwd(q, k, v, bias=None, causal=False, scale=None, seqlens=None,
-                  p_drop=0.0, seed=0, dtype=np.float64, return_probs=False, pos_offset=(0, 0, 0)):
+                  p_drop=0.0, seed=0, dtype=np.float64, return_probs=False, pos_offset=(0, 0, 0), kv_lens=None):
 	"""O [B,Sq,Hq,D] and LSE [B,Hq,Sq] (natural log) of exact attention.
 
 	q [B,Sq,Hq,D], k/v [B,Sk,Hkv,D].  Rows with no allowed key give O = 0 and
@@ -193,7 +197,7 @@ def attention_fwd(q, k, v, bias=None, causal=False, scale=None, seqlens=None,
 	B, Sq, Hq, D = q.shape
 	Sk, Hkv = k.shape[1], k.shape[2]
 	scale = (1.0 / math.sqrt(D)) if scale is None else scale
-	s, ok, r = _scores(q, k, bias, scale, causal, seqlens, dtype)
+	s, ok, r = _scores(q, k, bias, scale, causal, seqlens, dtype, kv_lens)
 	m = np.max(s, axis=-1, keepdims=True)
 	m_safe = np.where(np.isfinite(m), m, 0.0)
 	e = np.exp(s - m_safe)
@@ -213,7 +217,7 @@ def attention_fwd(q, k, v, bias=None, causal=False, scale=None, seqlens=None,
 
 
 def attention_bwd(q, k, v, dO, bias=None, causal=False, scale=None, seqlens=None,
-                  p_drop=0.0, seed=0, dtype=np.float64, pos_offset=(0, 0, 0)):
+                  p_drop=0.0, seed=0, dtype=np.float64, pos_offset=(0, 0, 0), kv_lens=None):
 	"""Analytic gradients (dQ, dK, dV) of sum(O * dO); FlashAttention-2 Algorithm 2,
 	the same five products as flash_attention_jax/_backward_jax.py:111-127, with
 	dK/dV summed over the q-heads of each KV group (_backward_triton.py:1156-1161).
@@ -221,7 +225,7 @@ def attention_bwd(q, k, v, dO, bias=None, causal=False, scale=None, seqlens=None
 	B, Sq, Hq, D = q.shape
 	Sk, Hkv = k.shape[1], k.shape[2]
 	scale = (1.0 / math.sqrt(D)) if scale is None else scale
-	o, lse, p, pd = attention_fwd(q, k, v, bias, causal, scale, seqlens, p_drop, seed, dtype, True, pos_offset)
+	o, lse, p, pd = attention_fwd(q, k, v, bias, causal, scale, seqlens, p_drop, seed, dtype, True, pos_offset, kv_lens)
 	r = Hq // Hkv
 	dOf = np.asarray(dO, dtype=dtype)
 	qf = np.asarray(q, dtype=dtype)

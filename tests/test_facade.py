@@ -83,6 +83,20 @@ def test_unbuilt_platforms_say_so():
 		create_flash_attention("tpu", "pallas")(q, q, q)
 
 
+def test_package_exports_the_names_of_the_reference():
+	"""jax_flash_attn2/__init__.py:23-35 of the reference: every public name exists here; the two pure-XLA
+	implementations are names that say they are not part of this package."""
+	import jax_flash_attn2 as pkg
+
+	for name in ("AttentionConfig", "Backend", "FlashAttention", "Platform", "create_flash_attention",
+	             "triton_flash_attention", "jax_flash_attention", "basic_attention_refrence"):
+		assert hasattr(pkg, name) and name in pkg.__all__, name
+	assert pkg.triton_flash_attention is pkg.hip_flash_attention
+	for fn in (pkg.jax_flash_attention, pkg.basic_attention_refrence):
+		with pytest.raises(NotImplementedError, match="HIP"):
+			fn(None, None, None)
+
+
 def test_kernel_head_dim_padding_rule():
 	torch = pytest.importorskip("torch")
 	from jax_flash_attn2 import _hip_op

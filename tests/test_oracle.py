@@ -175,6 +175,25 @@ def test_backward_identities():
 	assert np.allclose(dk, dk2.reshape(1, 12, 2, 2, 8).sum(3)) and np.allclose(dv, dv2.reshape(1, 12, 2, 2, 8).sum(3))
 
 
+def test_key_lengths_equal_an_explicit_key_mask():
+	"""kv_lens (key padding only) = -inf bias on the padded keys; rows and the causal offset stay as they are."""
+	rng = np.random.default_rng(11)
+	B, Sq, Sk, Hq, Hkv, D = 2, 10, 14, 4, 2, 8
+	q, k, v, dO = _rand(rng, B, Sq, Sk, Hq, Hkv, D)
+	lens = [9, 14]
+	big = np.zeros((B, 1, Sq, Sk))
+	big[0, :, :, 9:] = -1e30
+	for causal in (False, True):
+		o, lse = O.attention_fwd(q, k, v, causal=causal, kv_lens=lens)
+		o2, lse2 = O.attention_fwd(q, k, v, bias=big, causal=causal)
+		assert np.allclose(o, o2) and np.allclose(lse, lse2)
+		for a, b in zip(O.attention_bwd(q, k, v, dO, causal=causal, kv_lens=lens), O.attention_bwd(q, k, v, dO, bias=big, causal=causal)):
+			assert np.allclose(a, b)
+	# a length of zero: no key at all
+	o, lse = O.attention_fwd(q, k, v, kv_lens=[0, 14])
+	assert np.all(o[0] == 0) and np.all(np.isneginf(lse[0])) and np.all(np.isfinite(lse[1]))
+
+
 def test_blockwise_restatement_equals_closed_form():
 	rng = np.random.default_rng(7)
 	B, S, Hq, Hkv, D = 1, 256, 4, 2, 16

@@ -210,7 +210,7 @@ def test_rows_masked_entirely_by_finfo_min_bias_stay_finite():
 
 
 def test_boolean_4d_mask_through_the_facade():
-	"""A 4-D boolean mask is turned into the finfo.min bias of README.md:188 by the operator; also for Sq != Sk, where
+	"""A 4-D boolean mask acts as the finfo.min bias of README.md:188 (the kernels read the mask itself); also for Sq != Sk, where
 	the facade drops the reference's 2-D mask (flash_attention.py:239-242)."""
 	from jax_flash_attn2 import AttentionConfig, FlashAttention, Platform
 
@@ -225,6 +225,80 @@ def test_boolean_4d_mask_through_the_facade():
 		out = attn(_dev(q), _dev(k), _dev(v), attention_mask=_dev(mask))
 		err = float(np.abs(out.float().cpu().numpy() - o_ref).max())
 		assert err <= TOL_O[torch.bfloat16], f"4-D mask Sq{Sq} Sk{Sk}: O max-abs {err:.3e}"
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("mshape", [(2, 1), (1, 1), (2, 4), (1, 4)], ids=["bBh1", "b1h1", "bBhH", "b1hH"])
+def test_boolean_mask_operand_equals_the_finfo_min_bias(dtype, mshape):
+	"""A boolean mask handed over as one byte per position (fa2_params.bias_dtype = FA2_MASK_U8) against the oracle
+	given the bias where(mask, 0, finfo(dtype).min) of README.md:188 - forward and backward, broadcast over batch
+	and heads, ragged key counts, causal or not, including rows whose every key is masked (which that bias turns
+	into a plain average over all keys for bf16, and into the unmasked softmax for fp16, whose finfo.min does not
+	absorb the score)."""
+	B, Hq, Hkv = 2, 4, 2
+	for (Sq, Sk, D, causal) in ((160, 160, 128, False), (96, 203, 64, False), (130, 130, 64, True), (64, 96, 256, False)):
+		q, k, v, do, _ = make_inputs(B, Sq, Sk, Hq, Hkv, D, dtype, 31)
+		g = torch.Generator().manual_seed(9)
+		mask = torch.rand(*mshape, Sq, Sk, generator=g) < 0.6
+		if causal:
+			mask[..., 0] = True    # (or the first rows, which see few keys, would often have none left)
+		mask[..., 5, :] = False    # a row without any allowed key
+		mask[..., 0, 1:] = False   # rows with a single key
+		mask[..., 0, 0] = True
+		# (bf16: the logsumexp of a fully masked row is finfo.min + log(sum), which fp32 rounds to finfo.min - the
+		# backward of such a row is then off by the factor `sum`, with a finfo.min bias just the same; the row gets
+		# no incoming gradient here, as rows that attend to nothing do not in practice)
+		do[:, 5] = 0
+		bias = torch.where(mask, 0.0, float(torch.finfo(dtype).min)).to(dtype)
+		kw = dict(causal=causal)
+		o_ref, lse_ref = O.attention_fwd(f64(q), f64(k), f64(v), f64(bias), **kw)
+		g_ref = O.attention_bwd(f64(q), f64(k), f64(v), f64(do), f64(bias), **kw)
+		o, lse = op.fwd(_dev(q), _dev(k), _dev(v), _dev(mask), None, None, 0.0, causal, 0)
+		gr = op.bwd(_dev(q), _dev(k), _dev(v), o, lse, _dev(do), _dev(mask), None, None, 0.0, causal, 0)
+		what = f"mask {mshape} Sq{Sq} Sk{Sk} D{D} {dtype} causal={causal}"
+		# lse of a fully masked row sits near finfo.min: compare it relatively there
+		fin = lse_ref > -1e4
+		check_forward(o, torch.where(_dev(torch.from_numpy(fin)), lse, torch.zeros_like(lse)), o_ref, np.where(fin, lse_ref, 0.0), dtype, what)
+		lg = lse.cpu().numpy()
+		assert np.allclose(lg[~fin], lse_ref[~fin], rtol=1e-3), what
+		check_grads(gr, g_ref, what)
+		# the same numbers as the bias the mask stands for
+		o_b, lse_b = op.fwd(_dev(q), _dev(k), _dev(v), _dev(bias), None, None, 0.0, causal, 0)
+		assert float((o.float() - o_b.float()).abs().max()) <= 2.0 ** -7
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_key_lengths_with_bias_and_cross_lengths(causal):
+	"""fa2_params.kv_lens: per-batch key padding that, unlike the reference's 2-D mask, goes together with a bias and
+	with Sq != Sk.  Checked against explicit masking in the oracle; keys beyond the length get exactly zero gradient,
+	a length of zero leaves rows without keys (O = 0, lse = -inf)."""
+	for (B, Sq, Sk, Hq, Hkv, D, lens, bshape) in (
+		(3, 160, 160, 4, 2, 128, [160, 77, 1], (3, 1)),
+		(2, 100, 300, 4, 4, 64, [300, 130], None),
+		(4, 64, 200, 2, 1, 64, [0, 200, 64, 199], (1, 2)),
+		(2, 130, 130, 2, 2, 256, [129, 40], None),
+	):
+		bias_shape = None if bshape is None else (*bshape, Sq, Sk)
+		q, k, v, do, bias = make_inputs(B, Sq, Sk, Hq, Hkv, D, torch.bfloat16, 41, bias_shape)
+		kw = dict(causal=causal, kv_lens=lens)
+		o_ref, lse_ref = O.attention_fwd(f64(q), f64(k), f64(v), f64(bias), **kw)
+		g_ref = O.attention_bwd(f64(q), f64(k), f64(v), f64(do), f64(bias), **kw)
+		kl = torch.tensor(lens, dtype=torch.int32, device=DEV)
+		o, lse = op.fwd(_dev(q), _dev(k), _dev(v), _dev(bias), None, None, 0.0, causal, 0, kl)
+		gr = op.bwd(_dev(q), _dev(k), _dev(v), o, lse, _dev(do), _dev(bias), None, None, 0.0, causal, 0, kl)
+		what = f"kv_lens {lens} Sq{Sq} Sk{Sk} D{D} causal={causal} bias={bshape}"
+		check_forward(o, lse, o_ref, lse_ref, torch.bfloat16, what)
+		check_grads(gr, g_ref, what)
+		for b, n in enumerate(lens):
+			assert gr[1][b, n:].abs().max().item() == 0 and gr[2][b, n:].abs().max().item() == 0 if n < Sk else True
+	# through the differentiation rule
+	q, k, v, do, bias = make_inputs(2, 96, 96, 2, 2, 64, torch.bfloat16, 42, (2, 1, 96, 96))
+	kl = torch.tensor([50, 96], dtype=torch.int32, device=DEV)
+	qq = _dev(q).requires_grad_()
+	out = op.flash_attention(qq, _dev(k), _dev(v), bias=_dev(bias), causal=causal, kv_lens=kl)
+	out.backward(_dev(do))
+	g_ref = O.attention_bwd(f64(q), f64(k), f64(v), f64(do), f64(bias), causal=causal, kv_lens=[50, 96])
+	assert O.rel_l2(qq.grad.float().cpu().numpy(), g_ref[0]) <= 1e-2
 
 
 def test_mask_as_finfo_min_bias():
@@ -251,6 +325,28 @@ def test_mask_as_finfo_min_bias():
 def test_seqlens(causal):
 	_run_case(4, 256, 256, 4, 2, 128, torch.bfloat16, causal=causal, seqlens=[256, 100, 1, 0])
 	_run_case(3, 200, 200, 2, 2, 64, torch.float16, causal=causal, seqlens=[17, 200, 129])
+
+
+def test_2d_mask_is_applied_for_a_single_batch_row_too():
+	"""Intended difference from the reference: its GPU path only honours a 2-D attention_mask when the batch has more
+	than one row (`varlen_mode = attention_mask.shape[0] > 1`, _forward_triton.py:474-475, 498) and silently ignores
+	it for B == 1.  Here the mask always applies: keys beyond the valid length are masked, padded query rows give 0."""
+	B, S, H, D, n = 1, 96, 2, 64, 40
+	q, k, v, do, _ = make_inputs(B, S, S, H, H, D, torch.bfloat16, 21)
+	mask = torch.zeros(B, S, dtype=torch.int32)
+	mask[:, :n] = 1
+	qq, kk, vv = (_dev(t).requires_grad_() for t in (q, k, v))
+	out = op.flash_attention(qq, kk, vv, attention_mask=_dev(mask), causal=True)
+	out.backward(_dev(do))
+	o_ref, _ = O.attention_fwd(f64(q), f64(k), f64(v), causal=True, seqlens=[n])
+	g_ref = O.attention_bwd(f64(q), f64(k), f64(v), f64(do), causal=True, seqlens=[n])
+	got = out.detach().float().cpu().numpy()
+	assert np.abs(got - o_ref).max() <= TOL_O[torch.bfloat16]
+	assert np.abs(got[:, n:]).max() == 0.0 and np.abs(o_ref[:, n:]).max() == 0.0
+	check_grads((qq.grad, kk.grad, vv.grad), g_ref, "B == 1 with a 2-D mask")
+	# what the reference computes for this call (mask ignored) is something else
+	o_unmasked, _ = O.attention_fwd(f64(q), f64(k), f64(v), causal=True)
+	assert np.abs(o_unmasked[:, n:]).max() > 0.1
 
 
 @pytest.mark.parametrize("D", [64, 128, 256])
