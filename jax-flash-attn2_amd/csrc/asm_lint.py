@@ -8,7 +8,8 @@ the product runs.  The sources keep those distances by construction; this script
 assembly text the compiler emits for the same translation unit (`hipcc -S`, no binary is
 taken apart) and fails the build when a later compiler version, or an edit, breaks one.
 
-Rules, per kernel, in program-text order (a v_mfma between `;;#ASMSTART` and `;;#ASMEND`):
+Rules, per kernel, in program-text order along fall-through paths (the scan follows the text and
+forgets what is pending at an unconditional branch; a v_mfma between `;;#ASMSTART` and `;;#ASMEND`):
   R1  the product's C operand, when it is not also its destination, is not written by any
       instruction before one further v_mfma has been issued (or 7 wait states have passed):
       an 8-pass product reads C while it runs, and the hardware does not hold back a
@@ -125,6 +126,8 @@ def lint(path: str):
 				if is_mfma:
 					p["mfma"] += 1
 			pending = [p for p in pending if p["mfma"] < 2 and p["wait"] < max(R1_WAIT, R2_WAIT)]
+			if mn in ("s_branch", "s_endpgm", "s_setpc_b64"):
+				pending = []  # the next line of text is not reached from here
 			if is_mfma and in_asm and len(ops) >= 4:
 				dst, c = _regs(ops[0]), _regs(ops[3])
 				pending.append({"line": ln, "c": (c if c and c != dst else None), "dst": dst, "mfma": 0, "wait": 0})

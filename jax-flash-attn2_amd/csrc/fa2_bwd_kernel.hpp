@@ -84,13 +84,19 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	constexpr bool BIAS_LDS = BIAS && BIAS_T && 4 * TILE_BYTES + 4 * STAT_BYTES + 2 * BMQ * BN * 2 <= 160 * 1024 && D <= 128;
 	constexpr int BIAS_BYTES = BIAS_LDS ? BMQ * BN * 2 : 0;
 	static_assert(BN == 128, "bias tiles use the 128-element row geometry");
-	// Q[0] Q[1] dO[0] dO[1] | lse[0] lse[1] delta[0] delta[1] | bias[0] bias[1]
+	// Q[0] dO[0] Q[1] dO[1] | lse[0] lse[1] delta[0] delta[1] | bias[0] bias[1]
+	// (buffer 1 of each kind lies a power of two behind buffer 0: the per-lane read addresses below
+	// carry the buffer in that one bit and are flipped once per step, so that every read in the
+	// loop is register + immediate with no address arithmetic)
 	__shared__ __attribute__((aligned(1024))) char smem[4 * TILE_BYTES + 4 * STAT_BYTES + 2 * BIAS_BYTES];
 	FA2_LDS char* lds = (FA2_LDS char*)smem;
 	FA2_LDS char* stat = lds + 4 * TILE_BYTES;
 	FA2_LDS char* lds_bias = lds + 4 * TILE_BYTES + 4 * STAT_BYTES;
 
-	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+	const int tid = threadIdx.x, lane = tid & 63;
+	// the wave index as an explicitly scalar value: everything derived from it (tile bounds, loop trip counts,
+	// "nothing to do for this wave") then stays in scalar registers and scalar branches
+	const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int g = lane >> 5, c = lane & 31;
 	const int r = a.Hq / a.Hkv;
 	// dropout key: from the parameter block, or from device memory when the caller keeps it there
@@ -209,33 +215,27 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 			bload.load(lds_bias + (step & 1) * BIAS_BYTES, bb_, a.bias_sm, rows, tid, (a.Sk - n0) >> 3);
 		}
 	};
-	// per-row statistics of a tile: thread t < BMQ fetches lse, t in [BMQ, 2 BMQ) fetches delta
+	// per-row statistics of a tile: thread t < BMQ fetches lse, t in [BMQ, 2 BMQ) fetches delta.
+	// The value is only touched again in store_stat(), a whole step later: nothing here may wait for the load.
+	const int stat_row = tid % BMQ;
+	const float* stat_src = tid < BMQ ? a.lse : a.delta;
 	auto fetch_stat = [&](int step) -> float {
 		float x = 0.f;
 		if (tid < 2 * BMQ) {
 			int hq, m0;
 			decode_step(step, hq, m0);
-			int i = m0 + (tid % BMQ);
+			int i = m0 + stat_row;
 			i = i < a.Sq ? i : a.Sq - 1;
-			int64_t idx = ((int64_t)b * a.Hq + hq) * a.Sq + i;
-			if (tid < BMQ) {
-				x = a.lse[idx];
-				// FOLD: in units of the raw dot product (c1 of them make one log2 unit)
-				if constexpr (FOLD)
-					x *= inv_scale;
-				else if constexpr (!BIAS)
-					x *= kLog2e;
-			} else {
-				x = a.delta[idx];
-			}
-			if constexpr (FOLD) x = -x;
+			x = stat_src[((int64_t)b * a.Hq + hq) * a.Sq + i];
 		}
 		return x;
 	};
+	// lse in the units the elementwise stage wants, both negated where they start the chains
+	const float stat_mul = (tid < BMQ ? (FOLD ? inv_scale : (BIAS ? 1.f : kLog2e)) : 1.f) * (FOLD ? -1.f : 1.f);
 	auto store_stat = [&](float x, int buf) {
 		if (tid < 2 * BMQ) {
 			int which = tid / BMQ;
-			*(FA2_LDS float*)(stat + (2 * which + buf) * STAT_BYTES + (tid % BMQ) * 4) = x;
+			*(FA2_LDS float*)(stat + (2 * which + buf) * STAT_BYTES + stat_row * 4) = x * stat_mul;
 		}
 	};
 
@@ -256,6 +256,8 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		}
 	}
 
+	int soff = 16 * g;  // statistics: this half-wave's four rows of a quad (+ the buffer, flipped per step)
+
 	// bias tile (rows of 128 keys): this lane's 8-byte piece of rows 4 g + i16 / 4 (+ 8) at its wave's 32 keys
 	int boffq[2] = {0, 0};
 	if constexpr (BIAS_LDS) {
@@ -268,11 +270,8 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 
 	// One streamed tile of BMQ query rows of q-head hq.  MASKED = some (row, key)
 	// of this wave's 32 keys x BMQ rows is masked.
-	auto tile_body = [&](auto masked_tag, const FA2_LDS char* qt, const FA2_LDS char* dot, int buf, int hq, int m0)
-	                     __attribute__((always_inline)) {
+	auto tile_body = [&](auto masked_tag, int hq, int m0) __attribute__((always_inline)) {
 		constexpr bool MASKED = decltype(masked_tag)::value;
-		const FA2_LDS char* lse_s = stat + buf * STAT_BYTES;
-		const FA2_LDS char* del_s = stat + (2 + buf) * STAT_BYTES;
 		const char* bias_base = nullptr;
 		if constexpr (BIAS) {
 			int hb = a.bias_group ? hk : hq;
@@ -302,23 +301,22 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		f32x16 cstart[2];                 // start values of the chains of S and dP (inline-assembly path)
 		float bv[2][BIAS && !BIAS_LDS ? 16 : 1];  // [block parity]: bias values, fetched one stage ahead of their use
 		u32x2 bvr[2][BIAS_LDS ? 4 : 1];           // the same from LDS: [block parity][quad], 4 values of 16 bits
-		const FA2_LDS char* bt = lds_bias + buf * BIAS_BYTES;
 
 		// fragment of product j of A(qb): even j -> Q (S), odd j -> dO (dP), k-step j / 2
 		auto issue_A = [&](int qb, int j) __attribute__((always_inline)) {
-			const FA2_LDS char* base = ((j & 1) ? dot : qt) + poff[j >> 1] + qb * (32 * D * 2);
-			afr[(qb * NSLOT + j) % RING] = *(const FA2_LDS V8*)base;
+			// (poff carries the buffer; dO lies one tile behind Q)
+			afr[(qb * NSLOT + j) % RING] = *(const FA2_LDS V8*)(lds + poff[j >> 1] + ((j & 1) ? TILE_BYTES : 0) + qb * (32 * D * 2));
 		};
 		// fragment of product j of C(qb): half j / (2 DB); inside a half even -> dO^T (dV), odd -> Q^T (dK)
 		auto issue_C = [&](int qb, int j) __attribute__((always_inline)) {
 			int hf = j / (2 * DB), rr = j % (2 * DB), db = rr >> 1;
-			const FA2_LDS char* base = ((rr & 1) ? qt : dot) + qb * (32 * D * 2);
+			const FA2_LDS char* base = lds + ((rr & 1) ? 0 : TILE_BYTES) + qb * (32 * D * 2);
 			cfr[(qb * NSLOT + j) % RING] = lds_tr_issue_rt<D>(base + toff[db][0], base + toff[db][1], hf);
 		};
 		// statistics of rows 8 aa + 4 g .. + 3 of block qb
 		auto issue_stat = [&](int qb, int aa) __attribute__((always_inline)) {
-			lse4[aa] = *(const FA2_LDS f32x4*)(lse_s + (32 * qb + 8 * aa + 4 * g) * 4);
-			del4[aa] = *(const FA2_LDS f32x4*)(del_s + (32 * qb + 8 * aa + 4 * g) * 4);
+			lse4[aa] = *(const FA2_LDS f32x4*)(stat + soff + (32 * qb + 8 * aa) * 4);
+			del4[aa] = *(const FA2_LDS f32x4*)(stat + soff + 2 * STAT_BYTES + (32 * qb + 8 * aa) * 4);
 		};
 		// statistics of the quads whose phase 0 runs in slot j
 		auto issue_stat_for_slot = [&](int qb, int j) __attribute__((always_inline)) {
@@ -350,7 +348,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 				// quad j (rows 8 j + 4 g + e of the block, this lane's key): one transposed read
 				if (j < 4) {
 					typedef __attribute__((__vector_size__(4 * sizeof(short)))) short v4s;
-					v4s x = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FA2_LDS v4s*)(bt + boffq[j & 1] + (j >> 1) * (16 * 256) + qb * (32 * 256)));
+					v4s x = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FA2_LDS v4s*)(lds_bias + boffq[j & 1] + (j >> 1) * (16 * 256) + qb * (32 * 256)));
 					bvr[qb & 1][j] = __builtin_bit_cast(u32x2, x);
 				}
 			} else if constexpr (BIAS) {
@@ -644,7 +642,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	};
 
 	if (steps > 0) {
-		issue_tile(0, lds, lds + 2 * TILE_BYTES);
+		issue_tile(0, lds, lds + TILE_BYTES);
 		store_stat(fetch_stat(0), 0);
 	}
 
@@ -655,26 +653,36 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		__syncthreads();
 		float next_stat = 0.f;
 		const bool has_next = step + 1 < steps;
-		lds_pipeline_step(
-		    lds + buf * TILE_BYTES, lds + (2 + buf) * TILE_BYTES, lds + (buf ^ 1) * TILE_BYTES, lds + (2 + (buf ^ 1)) * TILE_BYTES,
-		    [&](FA2_LDS char* nq_, FA2_LDS char* ndo) {
-			    if (has_next) {
-				    // statistics first: loads return in order, so waiting for this small load later
-				    // does not wait for the tile copies issued after it
-				    next_stat = fetch_stat(step + 1);
-			    }
-			    if (has_next) issue_tile(step + 1, nq_, ndo);
-		    },
-		    [&](const FA2_LDS char* qt, const FA2_LDS char* dot) {
-			    int hq, m0;
-			    decode_step(step, hq, m0);
-			    if constexpr (decltype(masked_tag)::value) {
-				    // wave-uniform: nothing to do for (rows m0.., keys wn0..)?
-				    int last_row = m0 + BMQ - 1 < sq_eff - 1 ? m0 + BMQ - 1 : sq_eff - 1;
-				    if (wn0 >= sk_eff || (a.causal && wn0 > last_row + off)) return;
-			    }
-			    tile_body(masked_tag, qt, dot, buf, hq, m0);
-		    });
+		if (has_next) {
+			// statistics first: loads return in order, so waiting for this small load later
+			// does not wait for the tile copies issued after it
+			next_stat = fetch_stat(step + 1);
+			issue_tile(step + 1, lds + (buf ^ 1) * (2 * TILE_BYTES), lds + (buf ^ 1) * (2 * TILE_BYTES) + TILE_BYTES);
+		}
+		{
+			int hq, m0;
+			decode_step(step, hq, m0);
+			bool skip = false;
+			if constexpr (decltype(masked_tag)::value) {
+				// wave-uniform: nothing to do for (rows m0.., keys wn0..)?
+				int last_row = m0 + BMQ - 1 < sq_eff - 1 ? m0 + BMQ - 1 : sq_eff - 1;
+				skip = wn0 >= sk_eff || (a.causal && wn0 > last_row + off);
+			}
+			if (!skip) tile_body(masked_tag, hq, m0);
+		}
+		// the other buffers next time
+#pragma unroll
+		for (int ks = 0; ks < KS; ++ks) poff[ks] ^= 2 * TILE_BYTES;
+#pragma unroll
+		for (int db = 0; db < DB; ++db) {
+			toff[db][0] ^= 2 * TILE_BYTES;
+			toff[db][1] ^= 2 * TILE_BYTES;
+		}
+		soff ^= STAT_BYTES;
+		if constexpr (BIAS_LDS) {
+			boffq[0] ^= BIAS_BYTES;
+			boffq[1] ^= BIAS_BYTES;
+		}
 		if (has_next) store_stat(next_stat, buf ^ 1);
 	};
 	// Per q-head the streamed tiles are: tiles crossing this wave's causal diagonal
@@ -746,7 +754,10 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 	int mt, h, b;
 	decode_block(a, mt, h, b);
 	const int hk = h / (a.Hq / a.Hkv);
-	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+	const int tid = threadIdx.x, lane = tid & 63;
+	// the wave index as an explicitly scalar value: everything derived from it (tile bounds, loop trip counts,
+	// "nothing to do for this wave") then stays in scalar registers and scalar branches
+	const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int g = lane >> 5, c = lane & 31;
 	uint32_t drop_k0 = a.drop_k0, drop_k1 = a.drop_k1;
 	if constexpr (DROP) {

@@ -230,11 +230,13 @@ struct TileLoader {
 	uint32_t off[NIT];
 	int rows_state;  // the offsets clamp rows to [0, rows_state)
 	int cols_state;  // ... and 16-byte chunks of a row to [0, cols_state)
+	int wave_slot;   // byte offset of this wave's 64 x 16 bytes inside a piece (scalar)
 
 	// stride_bytes * ROWS must fit 31 bits (the launcher checks)
 	FA2_DEV void init(int64_t stride_bytes, int tid, int rows_valid = ROWS, int chunks_valid = CPR) {
 		rows_state = rows_valid;
 		cols_state = chunks_valid;
+		wave_slot = __builtin_amdgcn_readfirstlane((tid >> 6) << 10);
 #pragma unroll
 		for (int it = 0; it < NIT; ++it) {
 			int slot = it * NTHREADS + tid;
@@ -259,8 +261,7 @@ struct TileLoader {
 	}
 	// piece `it` (0 .. NIT-1) of the tile whose first row is at ub = uniform(address)
 	FA2_DEV void load_one(FA2_LDS char* tile, const char* ub, int it, int tid) const {
-		int wave_base = (tid >> 6) << 6;
-		lds_dma16_so(off[it], ub, tile + (it * NTHREADS + wave_base) * 16);
+		lds_dma16_so(off[it], ub, tile + it * NTHREADS * 16 + wave_slot);
 	}
 	// whole tile; rows at or beyond rows_valid are fetched from the last valid row, 16-byte chunks at or
 	// beyond chunks_valid from the last valid chunk of their row

@@ -148,7 +148,10 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 		decode_block(a, mt, h, b);
 	}
 	const int hk = h / (a.Hq / a.Hkv);
-	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+	const int tid = threadIdx.x, lane = tid & 63;
+	// the wave index as an explicitly scalar value: everything derived from it (tile bounds, loop trip counts,
+	// "nothing to do for this wave") then stays in scalar registers and scalar branches
+	const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int g = lane >> 5, c = lane & 31;
 	// dropout key: from the parameter block, or from device memory when the caller keeps it there
 	uint32_t drop_k0 = a.drop_k0, drop_k1 = a.drop_k1;
