@@ -910,6 +910,8 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 		if (bias_lds && ntiles > 0) bload.load(lds + 4 * TILE_BYTES, bias_base + (int64_t)m0 * a.bias_sm, a.bias_sm, brows, tid, a.Sk >> 3);
 	}
 
+	// (the offsets carry the buffer - K[1] / V[1] / bias[1] lie a power of two behind K[0] / V[0] / bias[0] -
+	// and are flipped after every tile, so that the reads need no address arithmetic in the loop)
 	int koff[KS];
 #pragma unroll
 	for (int ks = 0; ks < KS; ++ks) koff[ks] = tile_off<D>(c, 2 * ks + g);
@@ -926,7 +928,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 		}
 	}
 
-	auto tile_body = [&](auto masked_tag, const FA2_LDS char* kt, const FA2_LDS char* vt, const FA2_LDS char* bt, int n0) {
+	auto tile_body = [&](auto masked_tag, int n0) {
 		constexpr bool MASKED = decltype(masked_tag)::value;
 #pragma unroll
 		for (int kb = 0; kb < KB; ++kb) {
@@ -936,7 +938,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 				static_assert(!BIAS_LDS || QB == 1, "");
 #pragma unroll
 				for (int aa = 0; aa < 4; ++aa)
-					bvl[aa] = *(const FA2_LDS typename T::V4*)(bt + boff_lane + (((kb * 4 + aa) << 4) ^ bkey16));
+					bvl[aa] = *(const FA2_LDS typename T::V4*)(lds + 4 * TILE_BYTES + boff_lane + (((kb * 4 + aa) << 4) ^ bkey16));
 			} else if constexpr (BIAS) {
 #pragma unroll
 				for (int qb = 0; qb < QB; ++qb) {
@@ -955,10 +957,10 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 			__builtin_amdgcn_sched_barrier(0);
 #pragma unroll
 			for (int ks = 0; ks < KS; ++ks) {
-				V8 ka = *(const FA2_LDS V8*)(kt + koff[ks] + kb * (32 * D * 2));
+				V8 ka = *(const FA2_LDS V8*)(lds + koff[ks] + kb * (32 * D * 2));
 #pragma unroll
 				for (int qb = 0; qb < QB; ++qb) s[qb] = mfma32(ka, qf[qb][ks], s[qb]);
-				V8 va = *(const FA2_LDS V8*)(vt + koff[ks] + kb * (32 * D * 2));
+				V8 va = *(const FA2_LDS V8*)(lds + koff[ks] + 2 * TILE_BYTES + kb * (32 * D * 2));
 #pragma unroll
 				for (int qb = 0; qb < QB; ++qb) dp[qb] = mfma32(va, dof[qb][ks], (FOLD_DP && ks == 0) ? ndel16[qb] : dp[qb]);
 			}
@@ -977,7 +979,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 			// K^T fragments for dQ^T += K^T dS^T, issued ahead of the elementwise math
 			constexpr bool BOTH_EARLY = DB <= 4;
 			u32x4 kfr[2][DB];
-			const FA2_LDS char* kt_a = kt + kb * (32 * D * 2);
+			const FA2_LDS char* kt_a = lds + kb * (32 * D * 2);
 			auto issue_k = [&](int hf, u32x4(&dst)[DB]) {
 #pragma unroll
 				for (int db = 0; db < DB; ++db) dst[db] = lds_tr_issue_rt<D>(kt_a + toff[db][0], kt_a + toff[db][1], hf);
@@ -1036,27 +1038,29 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 		const int buf = t & 1;
 		wait_async_loads();
 		__syncthreads();
-		lds_pipeline_step(
-		    lds + buf * TILE_BYTES, lds + (2 + buf) * TILE_BYTES, lds + (buf ^ 1) * TILE_BYTES, lds + (2 + (buf ^ 1)) * TILE_BYTES,
-		    [&](FA2_LDS char* nk, FA2_LDS char* nv) {
-			    if (t + 1 < ntiles) {
-				    int n1 = n0 + BN;
-				    int rows = sk_eff - n1 < BN ? sk_eff - n1 : BN;
-				    kload.load(nk, kbase + (int64_t)n1 * a.k.ss, a.k.ss, rows, tid);
-				    vload.load(nv, vbase + (int64_t)n1 * a.v.ss, a.v.ss, rows, tid);
-				    if constexpr (BIAS_LDS) {
-					    if (bias_lds)
-						    bload.load(lds + 4 * TILE_BYTES + (buf ^ 1) * BIAS_BYTES, bias_base + (int64_t)m0 * a.bias_sm + (int64_t)n1 * 2,
-						               a.bias_sm, brows, tid, (a.Sk - n1) >> 3);
-				    }
-			    }
-		    },
-		    [&](const FA2_LDS char* kt, const FA2_LDS char* vt) {
-			    if constexpr (decltype(masked_tag)::value) {
-				    if (n0 > wave_jmax) return;  // whole tile masked for this wave (uniform)
-			    }
-			    tile_body(masked_tag, kt, vt, lds + 4 * TILE_BYTES + buf * BIAS_BYTES, n0);
-		    });
+		if (t + 1 < ntiles) {
+			int n1 = n0 + BN;
+			int rows = sk_eff - n1 < BN ? sk_eff - n1 : BN;
+			kload.load(lds + (buf ^ 1) * TILE_BYTES, kbase + (int64_t)n1 * a.k.ss, a.k.ss, rows, tid);
+			vload.load(lds + (2 + (buf ^ 1)) * TILE_BYTES, vbase + (int64_t)n1 * a.v.ss, a.v.ss, rows, tid);
+			if constexpr (BIAS_LDS) {
+				if (bias_lds)
+					bload.load(lds + 4 * TILE_BYTES + (buf ^ 1) * BIAS_BYTES, bias_base + (int64_t)m0 * a.bias_sm + (int64_t)n1 * 2,
+					           a.bias_sm, brows, tid, (a.Sk - n1) >> 3);
+			}
+		}
+		bool skip = false;
+		if constexpr (decltype(masked_tag)::value) skip = n0 > wave_jmax;  // whole tile masked for this wave (uniform)
+		if (!skip) tile_body(masked_tag, n0);
+		// the other buffers next time
+#pragma unroll
+		for (int ks = 0; ks < KS; ++ks) koff[ks] ^= TILE_BYTES;
+#pragma unroll
+		for (int db = 0; db < DB; ++db) {
+			toff[db][0] ^= TILE_BYTES;
+			toff[db][1] ^= TILE_BYTES;
+		}
+		if constexpr (BIAS_LDS) boff_lane ^= BIAS_BYTES;
 	};
 	// Tiles that lie entirely below every row's last allowed key need no mask.  They
 	// run in a loop of their own, so that the steady-state loop is a single

@@ -310,7 +310,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 		bload.init(a.bias_sm, tid, brows);
 		// this lane's row of the tile: byte offset of its chunk 0 (+ 8 bytes for the upper half-wave) and swizzle key
 		int row = w * (QB * 32) + c;
-		boff_lane = row * 128 + 8 * g;
+		boff_lane = row * 128 + 8 * g + (t_begin & 1) * BIAS_BYTES;
 		bkey16 = swz<64>(row) << 4;
 		if (bias_lds && ntiles > t_begin)
 			bload.load(lds + 4 * TILE_BYTES + (t_begin & 1) * BIAS_BYTES, bias_base + (int64_t)m0 * a.bias_sm + (int64_t)t_begin * BN * 2,
@@ -321,9 +321,12 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 	// read in the loop is base + register + immediate.
 	//   K fragment (ks):      row c (+32 kb), chunk 2ks+g
 	//   V fragment (kk, db):  rows 16kk + 4g + (lane&15)/4 (+8), 8 bytes at column 32db + 16((lane>>4)&1) + 4(lane&3)
+	// The offsets carry the buffer (K[1] / V[1] / bias[1] lie a power of two behind K[0] / V[0] / bias[0])
+	// and are flipped after every tile, so that the reads need no address arithmetic in the loop.
+	const int buf0 = t_begin & 1;
 	int koff[KS];
 #pragma unroll
-	for (int ks = 0; ks < KS; ++ks) koff[ks] = tile_off<D>(c, 2 * ks + g);
+	for (int ks = 0; ks < KS; ++ks) koff[ks] = tile_off<D>(c, 2 * ks + g) + buf0 * TILE_BYTES;
 	int voff[DB][2];
 	{
 		int i16 = lane & 15;
@@ -332,13 +335,13 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 #pragma unroll
 		for (int db = 0; db < DB; ++db) {
 			int col = 32 * db + vcol;
-			voff[db][0] = tile_off<D>(vrow, col >> 3) + ((col & 4) << 1);
-			voff[db][1] = tile_off<D>(vrow + 8, col >> 3) + ((col & 4) << 1);
+			voff[db][0] = tile_off<D>(vrow, col >> 3) + ((col & 4) << 1) + (2 + buf0) * TILE_BYTES;
+			voff[db][1] = tile_off<D>(vrow + 8, col >> 3) + ((col & 4) << 1) + (2 + buf0) * TILE_BYTES;
 		}
 	}
 
 	// One K/V tile.  MASKED = some element of the tile is masked for this wave.
-	auto tile_body = [&](auto masked_tag, const FA2_LDS char* kt, const FA2_LDS char* vt, const FA2_LDS char* bt, int n0) {
+	auto tile_body = [&](auto masked_tag, int n0) {
 		constexpr bool MASKED = decltype(masked_tag)::value;
 		// bias tile, fetched ahead of the matrix products
 		f32x4 bv[BIAS ? KB : 1][BIAS ? QB : 1][4];
@@ -348,7 +351,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 			for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
 				for (int aa = 0; aa < 4; ++aa) {
-					typename T::V4 x = *(const FA2_LDS typename T::V4*)(bt + boff_lane + (((kb * 4 + aa) << 4) ^ bkey16));
+					typename T::V4 x = *(const FA2_LDS typename T::V4*)(lds + 4 * TILE_BYTES + boff_lane + (((kb * 4 + aa) << 4) ^ bkey16));
 					bv[kb][0][aa] = __builtin_convertvector(x, f32x4);
 				}
 		} else if constexpr (BIAS) {
@@ -379,7 +382,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 			for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
 				for (int kb = 0; kb < KB; ++kb) {
-					V8 kf = *(const FA2_LDS V8*)(kt + koff[ks] + kb * (32 * D * 2));
+					V8 kf = *(const FA2_LDS V8*)(lds + koff[ks] + kb * (32 * D * 2));
 #pragma unroll
 					for (int qb = 0; qb < QB; ++qb) s[kb][qb] = mfma32(kf, qf[qb][ks], s[kb][qb]);
 				}
@@ -411,7 +414,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 			for (int f = 0; f < FPB; ++f)
 #pragma unroll
 				for (int db = 0; db < DB; ++db) {
-					dst[f * DB + db] = lds_tr_issue_rt<D>(vt + voff[db][0], vt + voff[db][1], BI * FPB + f);
+					dst[f * DB + db] = lds_tr_issue_rt<D>(lds + voff[db][0], lds + voff[db][1], BI * FPB + f);
 				}
 		};
 
@@ -615,27 +618,29 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 		const int buf = t & 1;
 		wait_async_loads();
 		__syncthreads();
-		lds_pipeline_step(
-		    lds + buf * TILE_BYTES, lds + (2 + buf) * TILE_BYTES, lds + (buf ^ 1) * TILE_BYTES, lds + (2 + (buf ^ 1)) * TILE_BYTES,
-		    [&](FA2_LDS char* nk, FA2_LDS char* nv) {
-			    if (t + 1 < ntiles) {
-				    int n1 = n0 + BN;
-				    int rows = sk_eff - n1 < BN ? sk_eff - n1 : BN;
-				    kload.load(nk, kbase + (int64_t)n1 * a.k.ss, a.k.ss, rows, tid);
-				    vload.load(nv, vbase + (int64_t)n1 * a.v.ss, a.v.ss, rows, tid);
-				    if constexpr (BIAS_LDS) {
-					    if (bias_lds)
-						    bload.load(lds + 4 * TILE_BYTES + (buf ^ 1) * BIAS_BYTES, bias_base + (int64_t)m0 * a.bias_sm + (int64_t)n1 * 2,
-						               a.bias_sm, brows, tid, (a.Sk - n1) >> 3);
-				    }
-			    }
-		    },
-		    [&](const FA2_LDS char* kt, const FA2_LDS char* vt) {
-			    if constexpr (decltype(masked_tag)::value) {
-				    if (n0 > wave_jmax) return;  // whole tile masked for this wave (uniform)
-			    }
-			    tile_body(masked_tag, kt, vt, lds + 4 * TILE_BYTES + buf * BIAS_BYTES, n0);
-		    });
+		if (t + 1 < ntiles) {
+			int n1 = n0 + BN;
+			int rows = sk_eff - n1 < BN ? sk_eff - n1 : BN;
+			kload.load(lds + (buf ^ 1) * TILE_BYTES, kbase + (int64_t)n1 * a.k.ss, a.k.ss, rows, tid);
+			vload.load(lds + (2 + (buf ^ 1)) * TILE_BYTES, vbase + (int64_t)n1 * a.v.ss, a.v.ss, rows, tid);
+			if constexpr (BIAS_LDS) {
+				if (bias_lds)
+					bload.load(lds + 4 * TILE_BYTES + (buf ^ 1) * BIAS_BYTES, bias_base + (int64_t)m0 * a.bias_sm + (int64_t)n1 * 2,
+					           a.bias_sm, brows, tid, (a.Sk - n1) >> 3);
+			}
+		}
+		bool skip = false;
+		if constexpr (decltype(masked_tag)::value) skip = n0 > wave_jmax;  // whole tile masked for this wave (uniform)
+		if (!skip) tile_body(masked_tag, n0);
+		// the other buffers next time
+#pragma unroll
+		for (int ks = 0; ks < KS; ++ks) koff[ks] ^= TILE_BYTES;
+#pragma unroll
+		for (int db = 0; db < DB; ++db) {
+			voff[db][0] ^= TILE_BYTES;
+			voff[db][1] ^= TILE_BYTES;
+		}
+		if constexpr (BIAS_LDS) boff_lane ^= BIAS_BYTES;
 	};
 	// Tiles that lie entirely below every row's last allowed key need no mask.  They
 	// run in a loop of their own, so that the steady-state loop is a single
