@@ -16,6 +16,14 @@ forgets what is pending at an unconditional branch; a v_mfma between `;;#ASMSTAR
       vector-ALU write to those registers;
   R2  the product's destination is not read by anything but a v_mfma C operand before two
       further v_mfma have been issued (or 11 wait states have passed).
+  R3  (over the kernel's control-flow graph, not the text order; every v_mfma, also the compiler's own)
+      no register of a matrix product's operands is read at a point that some path from the kernel's
+      entry reaches without writing it.  Seen with this compiler: a four-register operand spilled as
+      three registers to scratch memory plus one kept in a spare accumulation register, and reloaded
+      as three registers only - the product then read a stale fourth.  The build switches that kind of
+      spill off (-mllvm -amdgpu-spill-vgpr-to-agpr=0); this rule is the check that no operand is left
+      partly unwritten.  (Other instructions are not checked: under a divergent branch the compiler
+      legitimately reads registers that are only written for the lanes that use them.)
 A wait state is one instruction; `s_nop N` counts N + 1.
 
 Usage: asm_lint.py FILE.s [FILE.s ...]   (exit status 1 and one line per violation)
@@ -63,7 +71,8 @@ def _writes(mn: str, ops):
 		return set()
 	if mn.startswith(("v_swap", "v_permlane")):
 		return _regs(ops[0]) | (_regs(ops[1]) if len(ops) > 1 else set())
-	if mn.startswith(("v_", "ds_read", "ds_load", "global_load", "buffer_load", "flat_load", "scratch_load")):
+	if mn.startswith(("v_", "ds_read", "ds_load", "ds_bpermute", "ds_permute", "ds_swizzle", "global_load", "buffer_load", "flat_load",
+	                  "scratch_load")):
 		return _regs(ops[0])
 	return set()
 
@@ -134,6 +143,117 @@ def lint(path: str):
 	return problems
 
 
+_TARGET = re.compile(r"^(s_cbranch_\w+|s_branch)\s+(\S+)")
+_BLOCK = re.compile(r"^(\.L[\w$]+):")
+
+
+def _bit(reg):
+	return 1 << (reg[1] + (512 if reg[0] == "a" else 0))
+
+
+def _mask(regs):
+	m = 0
+	for r in regs:
+		m |= _bit(r)
+	return m
+
+
+def lint_defined(path: str):
+	"""Rule R3: definite assignment of vector registers over each kernel's control-flow graph."""
+	problems = []
+	kernels = []  # (name, [(ln, text)])
+	cur = None
+	with open(path) as f:
+		for ln, raw in enumerate(f, 1):
+			s = raw.strip()
+			m = _LABEL.match(s)
+			if m:
+				cur = (m.group(1), [])
+				kernels.append(cur)
+				continue
+			if cur is None:
+				continue
+			if s.startswith(".Lfunc_end"):
+				cur = None
+				continue
+			cur[1].append((ln, s))
+	for name, lines in kernels:
+		# basic blocks: a label starts one, a branch or the end of the program ends one
+		blocks = []  # dict: label, insts [(ln, text, reads, writes)], succ labels, falls
+		blk = {"label": None, "insts": [], "succ": [], "falls": True}
+		for ln, s in lines:
+			mb = _BLOCK.match(s)
+			if mb:
+				if blk["insts"] or blk["label"] is not None:
+					blocks.append(blk)
+				blk = {"label": mb.group(1), "insts": [], "succ": [], "falls": True}
+				continue
+			mn, ops = _split(s)
+			if mn is None:
+				continue
+			blk["insts"].append((ln, s, _mask(_reads(mn, ops)) if mn.startswith("v_mfma") else 0, _mask(_writes(mn, ops))))
+			mt = _TARGET.match(s)
+			if mt or mn in ("s_endpgm", "s_setpc_b64"):
+				if mt:
+					blk["succ"].append(mt.group(2))
+				blk["falls"] = bool(mt) and mt.group(1) != "s_branch"
+				blocks.append(blk)
+				blk = {"label": None, "insts": [], "succ": [], "falls": True}
+		if blk["insts"] or blk["label"] is not None:
+			blocks.append(blk)
+		if not blocks:
+			continue
+		index = {b["label"]: i for i, b in enumerate(blocks) if b["label"] is not None}
+		preds = [[] for _ in blocks]
+		for i, b in enumerate(blocks):
+			for t in b["succ"]:
+				if t in index:
+					preds[index[t]].append(i)
+			if b["falls"] and i + 1 < len(blocks):
+				preds[i + 1].append(i)
+		full = (1 << 1024) - 1
+		gen = []
+		for b in blocks:
+			g = 0
+			for _, _, _, w in b["insts"]:
+				g |= w
+			gen.append(g)
+		out = [full] * len(blocks)
+		entry = _bit(("v", 0))
+		changed = True
+		while changed:
+			changed = False
+			for i in range(len(blocks)):
+				if i == 0:
+					inn = entry
+				else:
+					inn = full
+					for p in preds[i]:
+						inn &= out[p]
+					if not preds[i]:
+						inn = full  # unreachable
+				o = inn | gen[i]
+				if o != out[i]:
+					out[i] = o
+					changed = True
+		reported = 0
+		for i, b in enumerate(blocks):
+			if i == 0:
+				have = entry
+			else:
+				have = full
+				for p in preds[i]:
+					have &= out[p]
+			for ln, s, r, w in b["insts"]:
+				miss = r & ~have & ~reported
+				if miss:
+					reported |= miss
+					names = [("a%d" % (k - 512)) if k >= 512 else ("v%d" % k) for k in range(1024) if (miss >> k) & 1]
+					problems.append(f"{path}:{ln}: {name}: R3: `{s}` reads {', '.join(names)}, unwritten on some path from the entry")
+				have |= w
+	return problems
+
+
 def main(argv):
 	if len(argv) < 2:
 		print(__doc__)
@@ -141,6 +261,7 @@ def main(argv):
 	bad = []
 	for path in argv[1:]:
 		bad += lint(path)
+		bad += lint_defined(path)
 	for b in bad:
 		print(b)
 	if bad:
