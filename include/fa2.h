@@ -122,6 +122,14 @@ typedef struct fa2_params {
 	 * batch that also carries a bias); key tiles beyond the length are skipped, not
 	 * masked.  A row left without any allowed key gives O = 0 and lse = -inf.       */
 	const int32_t* kv_lens; /* [B] int32 on device, NULL = all Sk keys     */
+
+	/* Optional sliding window (has_window != 0), the window_size of the reference's naive
+	 * attention (refrence_call.py:32,55-75): query row i attends to keys
+	 *   i + (Sk - Sq) - window_left  ..  i + (Sk - Sq) + window_right
+	 * where a negative bound means no bound on that side.  `causal` sets the right bound to 0
+	 * (refrence_call.py:36-37).  A row left without any key gives O = 0 and lse = -inf
+	 * (the reference zeroes such rows, :80-82).  Key tiles outside the window are skipped.  */
+	int32_t has_window, window_left, window_right;
 } fa2_params;
 
 /* sizeof(fa2_params) in the first version of this header: up to and including scratch_bytes */

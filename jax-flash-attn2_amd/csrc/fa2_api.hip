@@ -137,6 +137,9 @@ void fill(const fa2_params* p, KArgs& a) {
 	a.Hq = p->Hq;
 	a.Hkv = p->Hkv;
 	a.causal = p->causal ? 1 : 0;
+	// causal caps the right bound at 0, as the reference does (refrence_call.py:36-37)
+	a.win_left = p->has_window && p->window_left >= 0 ? p->window_left : -1;
+	a.win_right = p->causal ? 0 : (p->has_window && p->window_right >= 0 ? p->window_right : -1);
 	a.scale = p->scale;
 	a.drop_k0 = (uint32_t)(p->seed & 0xFFFFFFFFull);
 	a.drop_k1 = (uint32_t)(p->seed >> 32);
@@ -228,7 +231,7 @@ int fa2_fwd(const fa2_params* p, void* hip_stream) {
 	KArgs a;
 	fill(p, a);
 	// optional scratch: with enough of it a short query over many keys runs split over key ranges
-	size_t need = fa2_fwd_scratch_bytes(p);
+	size_t need = p->has_window ? 0 : fa2_fwd_scratch_bytes(p);  // (the split forward knows no window)
 	if (need && p->scratch && ((uintptr_t)p->scratch & 255) == 0 && p->scratch_bytes >= need) {
 		a.nsplit = fwd_split_plan(p, &a.split_len);
 		a.pack_gqa = fwd_pack_gqa(p) ? 1 : 0;

@@ -170,13 +170,21 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 #pragma unroll
 		for (int i = 0; i < 16; ++i) dk[db][i] = dv[db][i] = 0.f;
 
+	// Row i may look at keys i + off - win_left .. i + off + win_right (each bound only when >= 0; causal is
+	// win_right = 0), so key j is seen by rows j - off - win_right .. j - off + win_left.
+	const int wr = a.win_right, wl = a.win_left;
 	// query tiles that see at least one key of this workgroup
 	int q_lo = 0;
-	if (a.causal) {
-		int first = n0 - off;  // first row allowed to see key n0
+	if (wr >= 0) {
+		int first = n0 - off - wr;  // first row allowed to see key n0
 		q_lo = first > 0 ? first / BMQ : 0;
 	}
 	int q_hi = (sq_eff + BMQ - 1) / BMQ;  // exclusive
+	if (wl >= 0) {
+		int last = n0 + BN - 1 - off + wl;  // last row allowed to see the workgroup's last key
+		int e = last >= 0 ? last / BMQ + 1 : 0;
+		q_hi = e < q_hi ? e : q_hi;
+	}
 	if (n0 >= sk_eff) q_hi = q_lo;
 	const int nq = q_hi > q_lo ? q_hi - q_lo : 0;
 	const int steps = nq * r;
@@ -459,7 +467,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 						float p = exp2_fast(bx[q][e]);
 						if constexpr (MASKED) {
 							int row = m0 + 32 * qb + 8 * q + 4 * g + e;
-							bool ok = row < sq_eff && jcol < sk_eff && (!a.causal || jcol <= row + off);
+							bool ok = row < sq_eff && jcol < sk_eff && (wr < 0 || jcol <= row + off + wr) && (wl < 0 || jcol >= row + off - wl);
 							p = ok ? p : 0.f;
 						}
 						bx[q][e] = p;
@@ -498,7 +506,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 					float p = exp2_fast(bx[q][e]);
 					int row = m0 + 32 * qb + 8 * q + 4 * g + e;
 					if constexpr (MASKED) {
-						bool ok = row < sq_eff && jcol < sk_eff && (!a.causal || jcol <= row + off);
+						bool ok = row < sq_eff && jcol < sk_eff && (wr < 0 || jcol <= row + off + wr) && (wl < 0 || jcol >= row + off - wl);
 						p = ok ? p : 0.f;
 					}
 					bx[q][e] = p;
@@ -666,7 +674,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 			if constexpr (decltype(masked_tag)::value) {
 				// wave-uniform: nothing to do for (rows m0.., keys wn0..)?
 				int last_row = m0 + BMQ - 1 < sq_eff - 1 ? m0 + BMQ - 1 : sq_eff - 1;
-				skip = wn0 >= sk_eff || (a.causal && wn0 > last_row + off);
+				skip = wn0 >= sk_eff || (wr >= 0 && wn0 > last_row + off + wr) || (wl >= 0 && wn0 + 31 < m0 + off - wl);
 			}
 			if (!skip) tile_body(masked_tag, hq, m0);
 		}
@@ -685,17 +693,24 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		}
 		if (has_next) store_stat(next_stat, buf ^ 1);
 	};
-	// Per q-head the streamed tiles are: tiles crossing this wave's causal diagonal
-	// (masked), tiles entirely below it (no mask), and a ragged last tile (masked).
+	// Per q-head the streamed tiles are: tiles crossing this wave's causal diagonal / the window's
+	// right edge (masked), tiles entirely inside (no mask), and tiles on the window's left edge or a
+	// ragged last tile (masked).
 	// The unmasked tiles run in a loop of their own so that the steady state is a
 	// single straight-line body.
-	int i_diag = 0;  // first tile index (relative to q_lo) with no causal masking for this wave
-	if (a.causal) {
-		int first_clear = wn0 + 31 - off;  // rows >= this see all 32 keys of the wave
+	int i_diag = 0;  // first tile index (relative to q_lo) with no causal / right-edge masking for this wave
+	if (wr >= 0) {
+		int first_clear = wn0 + 31 - off - wr;  // rows >= this see all 32 keys of the wave
 		int tq = first_clear > 0 ? (first_clear + BMQ - 1) / BMQ : 0;
 		i_diag = tq - q_lo;
 	}
 	int i_full = sq_eff / BMQ - q_lo;  // tiles before this one lie entirely inside the valid rows
+	if (wl >= 0) {
+		// ... and entirely inside the left edge of the window: rows <= wn0 - off + win_left see even the wave's first key
+		int last_clear = wn0 - off + wl;
+		int e = last_clear >= 0 ? (last_clear + 1) / BMQ - q_lo : 0;
+		i_full = e < i_full ? e : i_full;
+	}
 	if (wn0 + 32 > sk_eff) i_diag = nq;  // ragged key block: always masked
 	i_diag = i_diag < 0 ? 0 : (i_diag > nq ? nq : i_diag);
 	i_full = i_full < i_diag ? i_diag : (i_full > nq ? nq : i_full);
@@ -783,25 +798,34 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 	const int m0 = mt * BM;
 	const int wm0 = m0 + w * (QB * 32);
 
+	// row i may look at keys i + off - win_left .. i + off + win_right (each bound only when >= 0; causal is win_right = 0)
+	const int wr = a.win_right, wl = a.win_left;
+	constexpr int kNoKey = -(1 << 30);
 	int kv_end = sk_eff;
-	if (a.causal) {
+	if (wr >= 0) {
 		int last_row = (m0 + BM - 1 < sq_eff - 1) ? m0 + BM - 1 : sq_eff - 1;
-		int e = last_row + off + 1;
+		int e = last_row + off + wr + 1;
 		kv_end = e < kv_end ? e : kv_end;
 	}
 	if (m0 >= sq_eff) kv_end = 0;
+	int t_begin = 0;
+	if (wl >= 0) {
+		int first_key = m0 + off - wl;  // first key the tile's first row sees
+		if (first_key > 0) t_begin = first_key / BN;
+	}
 	const int ntiles = kv_end > 0 ? (kv_end + BN - 1) / BN : 0;
 
-	int jmax[QB], qrow[QB];
+	int jmax[QB], jmin[QB], qrow[QB];
 	float lse_r[QB], del_r[QB];
 #pragma unroll
 	for (int qb = 0; qb < QB; ++qb) {
 		int i = wm0 + 32 * qb + c;
 		qrow[qb] = i;
 		int jm = sk_eff - 1;
-		if (a.causal) jm = (i + off < jm) ? i + off : jm;
+		if (wr >= 0) jm = (i + off + wr < jm) ? i + off + wr : jm;
 		if (i >= sq_eff) jm = -1;
 		jmax[qb] = jm;
+		jmin[qb] = wl >= 0 ? i + off - wl : kNoKey;
 		int ic = i < a.Sq ? i : a.Sq - 1;
 		int64_t idx = ((int64_t)b * a.Hq + h) * a.Sq + ic;
 		float l = a.lse[idx];
@@ -809,7 +833,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 		lse_r[qb] = BIAS ? l : l * kLog2e;
 		del_r[qb] = a.delta[idx];
 	}
-	int wave_jmin, wave_jmax;
+	int wave_jmin, wave_jmax, wave_lmin = kNoKey, wave_lmax = kNoKey;
 	{
 		int first = wm0, last = wm0 + QB * 32 - 1;
 		if (first >= sq_eff) {
@@ -818,9 +842,13 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 			wave_jmax = sk_eff - 1;
 			wave_jmin = sk_eff - 1;
 			int lastv = last < sq_eff - 1 ? last : sq_eff - 1;
-			if (a.causal) {
-				wave_jmax = (lastv + off < wave_jmax) ? lastv + off : wave_jmax;
-				wave_jmin = (first + off < wave_jmin) ? first + off : wave_jmin;
+			if (wr >= 0) {
+				wave_jmax = (lastv + off + wr < wave_jmax) ? lastv + off + wr : wave_jmax;
+				wave_jmin = (first + off + wr < wave_jmin) ? first + off + wr : wave_jmin;
+			}
+			if (wl >= 0) {
+				wave_lmin = first + off - wl;
+				wave_lmax = lastv + off - wl;
 			}
 			if (last >= sq_eff) wave_jmin = -1;
 		}
@@ -831,10 +859,11 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 	TileLoader<D, BN, NT> kload, vload;
 	kload.init(a.k.ss, tid);
 	vload.init(a.v.ss, tid);
-	if (ntiles > 0) {
-		int rows = sk_eff < BN ? sk_eff : BN;
-		kload.load(lds, kbase, a.k.ss, rows, tid);
-		vload.load(lds + 2 * TILE_BYTES, vbase, a.v.ss, rows, tid);
+	if (ntiles > t_begin) {
+		int nb = t_begin * BN, bsel = t_begin & 1;
+		int rows = sk_eff - nb < BN ? sk_eff - nb : BN;
+		kload.load(lds + bsel * TILE_BYTES, kbase + (int64_t)nb * a.k.ss, a.k.ss, rows, tid);
+		vload.load(lds + (2 + bsel) * TILE_BYTES, vbase + (int64_t)nb * a.v.ss, a.v.ss, rows, tid);
 	}
 
 	V8 qf[QB][KS], dof[QB][KS];
@@ -905,16 +934,18 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 		brows = a.Sq - m0 < BM ? a.Sq - m0 : BM;
 		bload.init(a.bias_sm, tid, brows);
 		int row = w * (QB * 32) + c;
-		boff_lane = row * 128 + 8 * g;
+		boff_lane = row * 128 + 8 * g + (t_begin & 1) * BIAS_BYTES;
 		bkey16 = swz<64>(row) << 4;
-		if (bias_lds && ntiles > 0) bload.load(lds + 4 * TILE_BYTES, bias_base + (int64_t)m0 * a.bias_sm, a.bias_sm, brows, tid, a.Sk >> 3);
+		if (bias_lds && ntiles > t_begin)
+			bload.load(lds + 4 * TILE_BYTES + (t_begin & 1) * BIAS_BYTES, bias_base + (int64_t)m0 * a.bias_sm + (int64_t)t_begin * BN * 2,
+			           a.bias_sm, brows, tid, (a.Sk - t_begin * BN) >> 3);
 	}
 
 	// (the offsets carry the buffer - K[1] / V[1] / bias[1] lie a power of two behind K[0] / V[0] / bias[0] -
 	// and are flipped after every tile, so that the reads need no address arithmetic in the loop)
 	int koff[KS];
 #pragma unroll
-	for (int ks = 0; ks < KS; ++ks) koff[ks] = tile_off<D>(c, 2 * ks + g);
+	for (int ks = 0; ks < KS; ++ks) koff[ks] = tile_off<D>(c, 2 * ks + g) + (t_begin & 1) * TILE_BYTES;
 	int toff[DB][2];
 	{
 		int i16 = lane & 15;
@@ -923,8 +954,8 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 #pragma unroll
 		for (int db = 0; db < DB; ++db) {
 			int col = 32 * db + tcol;
-			toff[db][0] = tile_off<D>(trow, col >> 3) + ((col & 4) << 1);
-			toff[db][1] = tile_off<D>(trow + 8, col >> 3) + ((col & 4) << 1);
+			toff[db][0] = tile_off<D>(trow, col >> 3) + ((col & 4) << 1) + (t_begin & 1) * TILE_BYTES;
+			toff[db][1] = tile_off<D>(trow + 8, col >> 3) + ((col & 4) << 1) + (t_begin & 1) * TILE_BYTES;
 		}
 	}
 
@@ -1006,7 +1037,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 							p = exp2_fast(__builtin_fmaf(s[qb][i], c1, -lse_r[qb]));
 						if constexpr (MASKED) {
 							int j = n0 + 32 * kb + 8 * aa + 4 * g + e;
-							p = j <= jmax[qb] ? p : 0.f;
+							p = (j <= jmax[qb] && j >= jmin[qb]) ? p : 0.f;
 						}
 						float dpe = dp[qb][i];
 						if constexpr (DROP) dpe = rnd[e] >= a.drop_thr ? dpe * a.drop_inv_keep : 0.f;
@@ -1050,7 +1081,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 			}
 		}
 		bool skip = false;
-		if constexpr (decltype(masked_tag)::value) skip = n0 > wave_jmax;  // whole tile masked for this wave (uniform)
+		if constexpr (decltype(masked_tag)::value) skip = n0 > wave_jmax || n0 + BN - 1 < wave_lmin;  // whole tile masked for this wave (uniform)
 		if (!skip) tile_body(masked_tag, n0);
 		// the other buffers next time
 #pragma unroll
@@ -1062,12 +1093,16 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 		}
 		if constexpr (BIAS_LDS) boff_lane ^= BIAS_BYTES;
 	};
-	// Tiles that lie entirely below every row's last allowed key need no mask.  They
-	// run in a loop of their own, so that the steady-state loop is a single
-	// straight-line body; the tiles on the causal diagonal / ragged end follow.
+	// Tiles that lie entirely inside every row's range of allowed keys need no mask.  They
+	// run in a loop of their own, so that the steady-state loop is a single straight-line
+	// body; the tiles on the window's left edge come before them, the tiles on the causal
+	// diagonal / right edge / ragged end after.
+	int t_lo = wave_lmax > 0 ? (wave_lmax + BN - 1) / BN : 0;
+	t_lo = t_lo < t_begin ? t_begin : (t_lo > ntiles ? ntiles : t_lo);
 	int t_full = (wave_jmin + 1) / BN;
-	t_full = t_full < 0 ? 0 : (t_full > ntiles ? ntiles : t_full);
-	for (int t = 0; t < t_full; ++t) step(std::false_type{}, t);
+	t_full = t_full < t_lo ? t_lo : (t_full > ntiles ? ntiles : t_full);
+	for (int t = t_begin; t < t_lo; ++t) step(std::true_type{}, t);
+	for (int t = t_lo; t < t_full; ++t) step(std::false_type{}, t);
 	for (int t = t_full; t < ntiles; ++t) step(std::true_type{}, t);
 
 	char* obase = a.dq.ptr + (int64_t)b * a.dq.sb + (int64_t)h * a.dq.sh;

@@ -178,11 +178,15 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 	const int m0 = mt * BM;
 	const int wm0 = m0 + w * (QB * 32);
 
+	// Row i may look at keys i + off - win_left .. i + off + win_right (each bound only when >= 0;
+	// causal is win_right = 0): the sliding window of refrence_call.py:55-75, bottom-right aligned.
+	const int wr = a.win_right, wl = a.win_left;
+	constexpr int kNoKey = -(1 << 30);
 	// keys this row tile can see (of this workgroup's range of keys)
 	int kv_end = sk_eff;
-	if (a.causal) {
+	if (wr >= 0) {
 		int last_row = (m0 + BM - 1 < sq_eff - 1) ? m0 + BM - 1 : sq_eff - 1;
-		int e = last_row + off + 1;
+		int e = last_row + off + wr + 1;
 		kv_end = e < kv_end ? e : kv_end;
 	}
 	if (m0 >= sq_eff) kv_end = 0;
@@ -193,11 +197,14 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 		kv_end = e < kv_end ? e : kv_end;
 		t_begin = kv_begin / BN;
 		if (kv_end <= kv_begin) kv_end = 0;
+	} else if (wl >= 0) {
+		int first_key = m0 + off - wl;  // first key the tile's first row sees
+		if (first_key > 0) t_begin = first_key / BN;
 	}
 	const int ntiles = kv_end > 0 ? (kv_end + BN - 1) / BN : 0;  // one past the last tile
 
-	// per-lane last allowed key for each of this lane's rows
-	int jmax[QB];
+	// per-lane first and last allowed key for each of this lane's rows
+	int jmax[QB], jmin[QB];
 	int qrow[QB];
 	int hl[QB];  // this lane's q-head
 #pragma unroll
@@ -216,12 +223,14 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 		}
 		qrow[qb] = i;
 		int jm = sk_eff - 1;
-		if (a.causal) jm = (i + off < jm) ? i + off : jm;
+		if (wr >= 0) jm = (i + off + wr < jm) ? i + off + wr : jm;
 		if (i >= sq_eff) jm = -1;
 		jmax[qb] = jm;
+		jmin[qb] = wl >= 0 ? i + off - wl : kNoKey;
 	}
-	// wave-uniform bounds of jmax over the wave's rows
-	int wave_jmin, wave_jmax;
+	// wave-uniform bounds over the wave's rows: wave_jmin / wave_jmax = smallest / largest last key,
+	// wave_lmin / wave_lmax = smallest / largest first key
+	int wave_jmin, wave_jmax, wave_lmin = kNoKey, wave_lmax = kNoKey;
 	{
 		int first = wm0, last = wm0 + QB * 32 - 1;
 		if (first >= sq_eff) {
@@ -230,9 +239,13 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 			wave_jmax = sk_eff - 1;
 			wave_jmin = sk_eff - 1;
 			int lastv = last < sq_eff - 1 ? last : sq_eff - 1;
-			if (a.causal) {
-				wave_jmax = (lastv + off < wave_jmax) ? lastv + off : wave_jmax;
-				wave_jmin = (first + off < wave_jmin) ? first + off : wave_jmin;
+			if (wr >= 0) {
+				wave_jmax = (lastv + off + wr < wave_jmax) ? lastv + off + wr : wave_jmax;
+				wave_jmin = (first + off + wr < wave_jmin) ? first + off + wr : wave_jmin;
+			}
+			if (wl >= 0) {
+				wave_lmin = first + off - wl;
+				wave_lmax = lastv + off - wl;
 			}
 			if (last >= sq_eff) wave_jmin = -1;
 		}
@@ -473,7 +486,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 								float p = exp2_fast(pv[e]);
 								if constexpr (MASKED) {
 									int j = n0 + 32 * kb + 8 * (2 * hf + (e >> 2)) + 4 * g + (e & 3);
-									p = j <= jmax[qb] ? p : 0.f;
+									p = (j <= jmax[qb] && j >= jmin[qb]) ? p : 0.f;
 								}
 								ls4[e & 3] += p;
 								pv[e] = p;
@@ -482,7 +495,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 						}
 					lt[qb] = (ls4[0] + ls4[1]) + (ls4[2] + ls4[3]);
 					// (a NaN sum - from inf or NaN inputs - also takes the other path, which propagates it)
-					over = over || !(lt[qb] <= kFastSum) || (mrow[qb] == -INFINITY && jmax[qb] >= n0);
+					over = over || !(lt[qb] <= kFastSum) || (mrow[qb] == -INFINITY && jmax[qb] >= n0 && jmin[qb] < n0 + BN);
 				}
 				slow = __builtin_amdgcn_ballot_w64(over) != 0;
 			}
@@ -499,7 +512,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 							float x = s[kb][qb][i];
 							if constexpr (MASKED) {
 								int j = n0 + 32 * kb + 8 * (i >> 2) + 4 * g + (i & 3);
-								x = j <= jmax[qb] ? x : -INFINITY;
+								x = (j <= jmax[qb] && j >= jmin[qb]) ? x : -INFINITY;
 							}
 							s[kb][qb][i] = x;
 							mx4[i & 3] = __builtin_fmaxf(mx4[i & 3], x);
@@ -544,7 +557,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 						float x = __builtin_fmaf(s[kb][qb][i], c1, bv[kb][qb][i >> 2][i & 3]);
 						if constexpr (MASKED) {
 							int j = n0 + 32 * kb + 8 * (i >> 2) + 4 * g + (i & 3);
-							x = j <= jmax[qb] ? x : -INFINITY;
+							x = (j <= jmax[qb] && j >= jmin[qb]) ? x : -INFINITY;
 						}
 						s[kb][qb][i] = x;
 						mx4[i & 3] = __builtin_fmaxf(mx4[i & 3], x);
@@ -630,7 +643,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 			}
 		}
 		bool skip = false;
-		if constexpr (decltype(masked_tag)::value) skip = n0 > wave_jmax;  // whole tile masked for this wave (uniform)
+		if constexpr (decltype(masked_tag)::value) skip = n0 > wave_jmax || n0 + BN - 1 < wave_lmin;  // whole tile masked for this wave (uniform)
 		if (!skip) tile_body(masked_tag, n0);
 		// the other buffers next time
 #pragma unroll
@@ -642,12 +655,16 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 		}
 		if constexpr (BIAS_LDS) boff_lane ^= BIAS_BYTES;
 	};
-	// Tiles that lie entirely below every row's last allowed key need no mask.  They
+	// Tiles that lie entirely inside every row's range of allowed keys need no mask.  They
 	// run in a loop of their own, so that the steady-state loop is a single
-	// straight-line body; the tiles on the causal diagonal / ragged end follow.
+	// straight-line body; the tiles on the window's left edge come before them, the tiles
+	// on the causal diagonal / right edge / ragged end after.
+	int t_lo = wave_lmax > 0 ? (wave_lmax + BN - 1) / BN : 0;  // first tile at or right of every row's first key
+	t_lo = t_lo < t_begin ? t_begin : (t_lo > ntiles ? ntiles : t_lo);
 	int t_full = (wave_jmin + 1) / BN;
-	t_full = t_full < t_begin ? t_begin : (t_full > ntiles ? ntiles : t_full);
-	for (int t = t_begin; t < t_full; ++t) step(std::false_type{}, t);
+	t_full = t_full < t_lo ? t_lo : (t_full > ntiles ? ntiles : t_full);
+	for (int t = t_begin; t < t_lo; ++t) step(std::true_type{}, t);
+	for (int t = t_lo; t < t_full; ++t) step(std::false_type{}, t);
 	for (int t = t_full; t < ntiles; ++t) step(std::true_type{}, t);
 
 	// epilogue: normalise, store O (lane: row c, four consecutive d per store) and LSE

@@ -26,7 +26,8 @@ struct KArgs {
 	const int32_t* seqlens;
 	const int32_t* kv_lens;  // [B]: keys at or beyond kv_lens[b] are masked (query rows unaffected)
 	int B, Sq, Sk, Hq, Hkv;
-	int causal;
+	int causal;      // (host side only: the kernels read win_right)
+	int win_left, win_right;  // row i sees keys i + off - win_left .. i + off + win_right; a negative bound is none; causal = win_right 0
 	float scale;
 	uint32_t drop_k0, drop_k1, drop_thr;
 	const uint32_t* seed_dev;  // when set: the Philox key (low word, high word) is read from device memory instead

@@ -67,7 +67,7 @@ def _usable(x: torch.Tensor) -> torch.Tensor:
 	return x
 
 
-def _fill_common(p, q, k, v, bias, seqlens, scale, p_drop, causal, seed, kv_lens=None):
+def _fill_common(p, q, k, v, bias, seqlens, scale, p_drop, causal, seed, kv_lens=None, window=None):
 	B, Sq, Hq, D = q.shape
 	Sk, Hkv = k.shape[1], k.shape[2]
 	p.dtype = _DTYPES[q.dtype]
@@ -89,6 +89,9 @@ def _fill_common(p, q, k, v, bias, seqlens, scale, p_drop, causal, seed, kv_lens
 		p.bias_group = 1 if (bias.shape[1] == Hkv and Hkv != Hq and bias.shape[1] != 1) else 0
 	if seqlens is not None:
 		p.seqlens = seqlens.data_ptr()
+	if window is not None:
+		left, right = window
+		p.has_window, p.window_left, p.window_right = 1, int(left), int(right)
 	if kv_lens is not None:
 		if kv_lens.dtype != torch.int32 or kv_lens.numel() != B or not kv_lens.is_contiguous():
 			raise ValueError("kv_lens must be a contiguous int32 tensor with one entry per batch row")
@@ -142,7 +145,8 @@ def _seqlens_from_mask(attention_mask, q):
 	return attention_mask.to(device=q.device).ne(0).sum(dim=1, dtype=torch.int32).contiguous()
 
 
-def fwd(q, k, v, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, causal=False, dropout_seed=None, kv_lens=None):
+def fwd(q, k, v, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, causal=False, dropout_seed=None, kv_lens=None,
+        window=None):
 	"""Returns (out [B,Sq,Hq,D] in q.dtype, lse [B,Hq,Sq] fp32 natural log)."""
 	lib = _lib.load()
 	D0 = q.shape[-1]
@@ -154,7 +158,7 @@ def fwd(q, k, v, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, 
 	out = torch.empty((B, Sq, Hq, D), dtype=q.dtype, device=q.device)
 	lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
 	p = _lib.new_params()
-	_fill_common(p, q, k, v, bias, seqlens, scale, dropout_prob, causal, dropout_seed, kv_lens)
+	_fill_common(p, q, k, v, bias, seqlens, scale, dropout_prob, causal, dropout_seed, kv_lens, window)
 	p.o = _t4(out)
 	p.lse = lse.data_ptr()
 	# short query over many keys: scratch lets the library split the keys over workgroups
@@ -168,7 +172,7 @@ def fwd(q, k, v, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, 
 
 
 def bwd(q, k, v, out, lse, dout, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, causal=False,
-        dropout_seed=None, kv_lens=None):
+        dropout_seed=None, kv_lens=None, window=None):
 	"""Returns (dq, dk, dv) in the dtypes of q, k, v; dk/dv summed over each KV group."""
 	lib = _lib.load()
 	D0 = q.shape[-1]
@@ -181,7 +185,7 @@ def bwd(q, k, v, out, lse, dout, bias=None, seqlens=None, softmax_scale=None, dr
 	dk = torch.empty_like(k, memory_format=torch.contiguous_format)
 	dv = torch.empty_like(v, memory_format=torch.contiguous_format)
 	p = _lib.new_params()
-	_fill_common(p, q, k, v, bias, seqlens, scale, dropout_prob, causal, dropout_seed, kv_lens)
+	_fill_common(p, q, k, v, bias, seqlens, scale, dropout_prob, causal, dropout_seed, kv_lens, window)
 	p.o = _t4(out)
 	p.lse = lse.data_ptr()
 	p.dout, p.dq, p.dk, p.dv = _t4(dout), _t4(dq), _t4(dk), _t4(dv)
@@ -213,7 +217,7 @@ class Plan:
 	enqueue kernels, nothing is allocated per call."""
 
 	def __init__(self, q, k, v, dout=None, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, causal=False,
-	             dropout_seed=None, kv_lens=None):
+	             dropout_seed=None, kv_lens=None, window=None):
 		self.lib = _lib.load()
 		self.q, self.k, self.v = _usable(q), _usable(k), _usable(v)
 		self.bias = _prep_bias(bias)
@@ -224,7 +228,7 @@ class Plan:
 		self.lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
 		p = self.params = _lib.new_params()
 		self.kv_lens = kv_lens
-		_fill_common(p, self.q, self.k, self.v, self.bias, seqlens, scale, dropout_prob, causal, dropout_seed, kv_lens)
+		_fill_common(p, self.q, self.k, self.v, self.bias, seqlens, scale, dropout_prob, causal, dropout_seed, kv_lens, window)
 		self.seed = dropout_seed  # (a device-resident seed must outlive the plan's calls)
 		p.o = _t4(self.out)
 		p.lse = self.lse.data_ptr()
@@ -261,18 +265,18 @@ class _FlashAttentionFn(torch.autograd.Function):
 	(_flash_attention.py:119-122).  Returns (dq, dk, dv) and None for everything else."""
 
 	@staticmethod
-	def forward(ctx, q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens=None):
-		out, lse = fwd(q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens)
+	def forward(ctx, q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens=None, window=None):
+		out, lse = fwd(q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens, window)
 		ctx.save_for_backward(q, k, v, bias, seqlens, out, lse, kv_lens)
-		ctx.cfg = (softmax_scale, dropout_prob, causal, dropout_seed)
+		ctx.cfg = (softmax_scale, dropout_prob, causal, dropout_seed, window)
 		return out
 
 	@staticmethod
 	def backward(ctx, dout):
 		q, k, v, bias, seqlens, out, lse, kv_lens = ctx.saved_tensors
-		softmax_scale, dropout_prob, causal, dropout_seed = ctx.cfg
-		dq, dk, dv = bwd(q, k, v, out, lse, dout, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens)
-		return dq, dk, dv, None, None, None, None, None, None, None
+		softmax_scale, dropout_prob, causal, dropout_seed, window = ctx.cfg
+		dq, dk, dv = bwd(q, k, v, out, lse, dout, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens, window)
+		return dq, dk, dv, None, None, None, None, None, None, None, None
 
 
 def flash_attention(
@@ -288,17 +292,20 @@ def flash_attention(
 	varlen_mode: bool = True,
 	*,
 	kv_lens=None,
+	window_size=None,
 ):
 	"""Same signature as the reference's `triton_flash_attention`
 	(_flash_attention.py:125-157).  `varlen_mode` is accepted for source
 	compatibility; padded batches are always handled in-kernel from per-row
 	lengths, never by packing.  `kv_lens` (keyword only, not in the reference):
 	int32 [B] number of valid keys per batch row - key padding that may be combined
-	with a bias and with Sq != Sk, which the 2-D attention_mask may not."""
+	with a bias and with Sq != Sk, which the 2-D attention_mask may not.  `window_size` =
+	(left, right) (keyword only): the sliding window of the reference's naive attention
+	(refrence_call.py:32,55-75); a negative bound is none, causal sets right = 0."""
 	del varlen_mode
 	if attention_mask is not None and attention_mask.dim() == 4:
 		assert bias is None, "Attention mask is not supported along with attention bias. Just use bias instead."
 		bias, attention_mask = _mask_operand(attention_mask, q), None
 	check_shapes(q, k, v, bias, attention_mask)
 	seqlens = _seqlens_from_mask(attention_mask, q)
-	return _FlashAttentionFn.apply(q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens)
+	return _FlashAttentionFn.apply(q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens, window_size)

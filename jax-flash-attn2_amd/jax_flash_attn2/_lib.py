@@ -59,6 +59,9 @@ class Fa2Params(ctypes.Structure):
 		("scratch_bytes", ctypes.c_uint64),
 		("seed_dev", ctypes.c_void_p),
 		("kv_lens", ctypes.c_void_p),
+		("has_window", ctypes.c_int32),
+		("window_left", ctypes.c_int32),
+		("window_right", ctypes.c_int32),
 	]
 
 

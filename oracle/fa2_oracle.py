@@ -127,7 +127,7 @@ def _expand_bias(bias, B, Hq, Hkv, Sq, Sk, dtype):
 	return np.broadcast_to(bias, (B, Hq, Sq, Sk))
 
 
-def allowed_mask(B, Sq, Sk, causal, seqlens=None, kv_lens=None):
+def allowed_mask(B, Sq, Sk, causal, seqlens=None, kv_lens=None, window=None):
 	"""allowed[b,i,j]: causal is bottom-right aligned (j <= i + Sk - Sq),
 	_forward_triton.py:127-132, refrence_call.py:66-67.  `seqlens[b]` is the
 	right-padded 2-D validity mask of the reference's GPU path reduced to a
@@ -135,12 +135,21 @@ def allowed_mask(B, Sq, Sk, causal, seqlens=None, kv_lens=None):
 	(_forward_triton.py:474-481,499-510,590-591).  With seqlens the causal
 	offset is 0 (it requires Sq == Sk).  `kv_lens[b]` (not in the reference:
 	plain key padding) masks keys j >= len only; rows and the causal offset
-	are untouched."""
+	are untouched.  `window` = (left, right) is the sliding window of the
+	naive reference (refrence_call.py:36-37,55-75): row i sees keys
+	i + Sk - Sq - left .. i + Sk - Sq + right, a negative bound meaning none, and
+	causal sets right = 0; unlike that code, right < 0 with left >= 0 is "no right
+	bound" here (there it would also hide the diagonal)."""
 	i = np.arange(Sq)[:, None]
 	j = np.arange(Sk)[None, :]
 	ok = np.ones((B, Sq, Sk), dtype=bool)
+	left, right = (-1, -1) if window is None else window
 	if causal:
-		ok &= (j <= i + (Sk - Sq))[None]
+		right = 0
+	if right >= 0:
+		ok &= (j <= i + (Sk - Sq) + right)[None]
+	if left >= 0:
+		ok &= (j >= i + (Sk - Sq) - left)[None]
 	if seqlens is not None:
 		L = np.asarray(seqlens).reshape(B, 1, 1)
 		ok &= (j[None] < L) & (i[None] < L)
@@ -169,7 +178,7 @@ def _ptx(p, x):
 	return np.swapaxes(np.matmul(np.swapaxes(p, 2, 3), _bh(x)), 1, 2)
 
 
-def _scores(q, k, bias, scale, causal, seqlens, dtype, kv_lens=None):
+def _scores(q, k, bias, scale, causal, seqlens, dtype, kv_lens=None, window=None):
 	B, Sq, Hq, D = q.shape
 	_, Sk, Hkv, _ = k.shape
 	if Hq % Hkv:
@@ -181,13 +190,13 @@ def _scores(q, k, bias, scale, causal, seqlens, dtype, kv_lens=None):
 	bb = _expand_bias(bias, B, Hq, Hkv, Sq, Sk, dtype)
 	if bb is not None:
 		s = s + bb
-	ok = allowed_mask(B, Sq, Sk, causal, seqlens, kv_lens)[:, None]
+	ok = allowed_mask(B, Sq, Sk, causal, seqlens, kv_lens, window)[:, None]
 	s = np.where(ok, s, -np.inf)
 	return s, ok, r
 
 
 def attention_fwd(q, k, v, bias=None, causal=False, scale=None, seqlens=None,
-                  p_drop=0.0, seed=0, dtype=np.float64, return_probs=False, pos_offset=(0, 0, 0), kv_lens=None):
+                  p_drop=0.0, seed=0, dtype=np.float64, return_probs=False, pos_offset=(0, 0, 0), kv_lens=None, window=None):
 	"""O [B,Sq,Hq,D] and LSE [B,Hq,Sq] (natural log) of exact attention.
 
 	q [B,Sq,Hq,D], k/v [B,Sk,Hkv,D].  Rows with no allowed key give O = 0 and
@@ -197,7 +206,7 @@ def attention_fwd(q, k, v, bias=None, causal=False, scale=None, seqlens=None,
 	B, Sq, Hq, D = q.shape
 	Sk, Hkv = k.shape[1], k.shape[2]
 	scale = (1.0 / math.sqrt(D)) if scale is None else scale
-	s, ok, r = _scores(q, k, bias, scale, causal, seqlens, dtype, kv_lens)
+	s, ok, r = _scores(q, k, bias, scale, causal, seqlens, dtype, kv_lens, window)
 	m = np.max(s, axis=-1, keepdims=True)
 	m_safe = np.where(np.isfinite(m), m, 0.0)
 	e = np.exp(s - m_safe)
@@ -217,7 +226,7 @@ def attention_fwd(q, k, v, bias=None, causal=False, scale=None, seqlens=None,
 
 
 def attention_bwd(q, k, v, dO, bias=None, causal=False, scale=None, seqlens=None,
-                  p_drop=0.0, seed=0, dtype=np.float64, pos_offset=(0, 0, 0), kv_lens=None):
+                  p_drop=0.0, seed=0, dtype=np.float64, pos_offset=(0, 0, 0), kv_lens=None, window=None):
 	"""Analytic gradients (dQ, dK, dV) of sum(O * dO); FlashAttention-2 Algorithm 2,
 	the same five products as flash_attention_jax/_backward_jax.py:111-127, with
 	dK/dV summed over the q-heads of each KV group (_backward_triton.py:1156-1161).
@@ -225,7 +234,7 @@ def attention_bwd(q, k, v, dO, bias=None, causal=False, scale=None, seqlens=None
 	B, Sq, Hq, D = q.shape
 	Sk, Hkv = k.shape[1], k.shape[2]
 	scale = (1.0 / math.sqrt(D)) if scale is None else scale
-	o, lse, p, pd = attention_fwd(q, k, v, bias, causal, scale, seqlens, p_drop, seed, dtype, True, pos_offset, kv_lens)
+	o, lse, p, pd = attention_fwd(q, k, v, bias, causal, scale, seqlens, p_drop, seed, dtype, True, pos_offset, kv_lens, window)
 	r = Hq // Hkv
 	dOf = np.asarray(dO, dtype=dtype)
 	qf = np.asarray(q, dtype=dtype)

@@ -194,6 +194,38 @@ def test_key_lengths_equal_an_explicit_key_mask():
 	assert np.all(o[0] == 0) and np.all(np.isneginf(lse[0])) and np.all(np.isfinite(lse[1]))
 
 
+def test_sliding_window_is_the_local_mask_of_the_naive_reference():
+	"""refrence_call.py:55-75 with no padding masks: a key is hidden iff col > min(row + sk - sq + right, sk) or
+	col < row + sk - sq - left (left >= 0), or col > row + sk - sq + right (left < 0); causal sets right = 0 (:36-37).
+	The oracle's window must be that mask wherever both bounds are given or only the right one; rows hidden
+	entirely give zeros (:80-82)."""
+	rng = np.random.default_rng(3)
+	for (Sq, Sk) in ((12, 12), (7, 15), (15, 7)):
+		row = np.arange(Sq)[:, None]
+		col = np.arange(Sk)[None, :]
+		for (left, right) in ((3, 0), (2, 2), (0, 0), (-1, 2), (-1, 0), (5, 1), (100, 100)):
+			if left < 0:
+				hidden = col > row + Sk - Sq + right
+			else:
+				hidden = (col > np.minimum(row + Sk - Sq + right, Sk)) | (col < row + Sk - Sq - left)
+			ok = O.allowed_mask(1, Sq, Sk, False, window=(left, right))[0]
+			assert np.array_equal(ok, ~hidden), (Sq, Sk, left, right)
+		assert np.array_equal(O.allowed_mask(1, Sq, Sk, True, window=(4, 9))[0], O.allowed_mask(1, Sq, Sk, False, window=(4, 0))[0])
+		assert np.array_equal(O.allowed_mask(1, Sq, Sk, True)[0], O.allowed_mask(1, Sq, Sk, False, window=(-1, 0))[0])
+	# equals an explicit -inf bias; fully hidden rows give O = 0
+	B, Sq, Sk, Hq, Hkv, D = 1, 9, 14, 2, 1, 4
+	q, k, v, dO = _rand(rng, B, Sq, Sk, Hq, Hkv, D)
+	ok = O.allowed_mask(B, Sq, Sk, False, window=(2, 1))
+	big = np.where(ok[:, None], 0.0, -1e30)
+	o, lse = O.attention_fwd(q, k, v, window=(2, 1))
+	o2, lse2 = O.attention_fwd(q, k, v, bias=big)
+	assert np.allclose(o, o2) and np.allclose(lse, lse2)
+	for a, b in zip(O.attention_bwd(q, k, v, dO, window=(2, 1)), O.attention_bwd(q, k, v, dO, bias=big)):
+		assert np.allclose(a, b)
+	o, lse = O.attention_fwd(q[:, :, :, :], k[:, :3], v[:, :3], window=(1, 0))  # Sq 9 > Sk 3: the first rows see nothing
+	assert np.all(o[:, :5] == 0) and np.all(np.isneginf(lse[..., :5]))
+
+
 def test_blockwise_restatement_equals_closed_form():
 	rng = np.random.default_rng(7)
 	B, S, Hq, Hkv, D = 1, 256, 4, 2, 16

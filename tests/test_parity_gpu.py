@@ -301,6 +301,45 @@ def test_key_lengths_with_bias_and_cross_lengths(causal):
 	assert O.rel_l2(qq.grad.float().cpu().numpy(), g_ref[0]) <= 1e-2
 
 
+@pytest.mark.parametrize("window", [(64, 0), (17, 5), (0, 0), (-1, 40), (200, -1), (130, 130), (1000, 1000)])
+def test_sliding_window(window):
+	"""The sliding window of the reference's naive attention (refrence_call.py:32,55-75), fused: forward and
+	backward against the oracle, self and cross lengths, with and without the causal flag (which caps the
+	right bound at 0), GQA, every head dim, with bias, dropout and key lengths; rows that the window leaves
+	without a key give zeros."""
+	cases = (
+		# B, Sq, Sk, Hq, Hkv, D, dtype, causal, bias heads, p
+		(2, 320, 320, 4, 2, 128, torch.bfloat16, False, None, 0.0),
+		(1, 200, 333, 4, 4, 64, torch.float16, False, None, 0.0),
+		(1, 333, 200, 2, 1, 64, torch.bfloat16, False, None, 0.0),
+		(2, 260, 260, 4, 2, 128, torch.bfloat16, True, None, 0.0),
+		(1, 192, 192, 2, 2, 256, torch.bfloat16, False, None, 0.0),
+		(2, 160, 224, 4, 2, 64, torch.bfloat16, False, (2, 1), 0.0),
+		(1, 192, 192, 4, 2, 128, torch.bfloat16, False, None, 0.2),
+	)
+	for (B, Sq, Sk, Hq, Hkv, D, dtype, causal, bh, p) in cases:
+		bias_shape = None if bh is None else (*bh, Sq, Sk)
+		q, k, v, do, bias = make_inputs(B, Sq, Sk, Hq, Hkv, D, dtype, 51, bias_shape)
+		kw = dict(causal=causal, window=window, p_drop=p, seed=9)
+		o_ref, lse_ref = O.attention_fwd(f64(q), f64(k), f64(v), f64(bias), **kw)
+		g_ref = O.attention_bwd(f64(q), f64(k), f64(v), f64(do), f64(bias), **kw)
+		o, lse = op.fwd(_dev(q), _dev(k), _dev(v), _dev(bias), None, None, p, causal, 9, None, window)
+		gr = op.bwd(_dev(q), _dev(k), _dev(v), o, lse, _dev(do), _dev(bias), None, None, p, causal, 9, None, window)
+		what = f"window {window} Sq{Sq} Sk{Sk} D{D} {dtype} causal={causal} bias={bh} p={p}"
+		check_forward(o, lse, o_ref, lse_ref, dtype, what)
+		check_grads(gr, g_ref, what)
+	# with key lengths, and through the differentiation rule
+	q, k, v, do, _ = make_inputs(2, 150, 150, 2, 2, 64, torch.bfloat16, 52)
+	kl = torch.tensor([150, 90], dtype=torch.int32, device=DEV)
+	qq = _dev(q).requires_grad_()
+	out = op.flash_attention(qq, _dev(k), _dev(v), kv_lens=kl, window_size=window)
+	out.backward(_dev(do))
+	o_ref, _ = O.attention_fwd(f64(q), f64(k), f64(v), kv_lens=[150, 90], window=window)
+	g_ref = O.attention_bwd(f64(q), f64(k), f64(v), f64(do), kv_lens=[150, 90], window=window)
+	assert np.abs(out.detach().float().cpu().numpy() - o_ref).max() <= TOL_O[torch.bfloat16]
+	check_grads((qq.grad,), (g_ref[0],), f"window {window} with key lengths")
+
+
 def test_mask_as_finfo_min_bias():
 	"""Boolean mask -> where(mask, 0, finfo.min) bias (the README recipe) must equal key-length masking."""
 	B, S, H, D = 2, 192, 4, 64
