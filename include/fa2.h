@@ -130,6 +130,11 @@ typedef struct fa2_params {
 	 * (refrence_call.py:36-37).  A row left without any key gives O = 0 and lse = -inf
 	 * (the reference zeroes such rows, :80-82).  Key tiles outside the window are skipped.  */
 	int32_t has_window, window_left, window_right;
+
+	/* Optional tanh soft-capping of the scores (> 0): softcap * tanh(scale q.k / softcap) takes the
+	 * place of scale q.k, before bias and masks, as in the reference's naive attention
+	 * (refrence_call.py:33,48-51); the backward carries the factor 1 - tanh^2.  0 = off.      */
+	float softcap;
 } fa2_params;
 
 /* sizeof(fa2_params) in the first version of this header: up to and including scratch_bytes */

@@ -62,6 +62,7 @@ int validate(const fa2_params* p, int which, bool own_scratch = false) {
 	if (p->D != 64 && p->D != 128 && p->D != 256) return FA2_EUNSUPPORTED;
 	if (!(p->p_drop >= 0.f && p->p_drop < 1.f)) return FA2_EINVAL_DROPOUT;
 	if (!isfinite(p->scale) || !(p->scale > 0.f)) return FA2_EINVAL_SHAPE;
+	if (!isfinite(p->softcap) || p->softcap < 0.f) return FA2_EINVAL_SHAPE;
 	int rc;
 	if ((rc = check_tensor(p->q, true))) return rc;
 	if ((rc = check_tensor(p->k, true))) return rc;
@@ -141,6 +142,8 @@ void fill(const fa2_params* p, KArgs& a) {
 	a.win_left = p->has_window && p->window_left >= 0 ? p->window_left : -1;
 	a.win_right = p->causal ? 0 : (p->has_window && p->window_right >= 0 ? p->window_right : -1);
 	a.scale = p->scale;
+	a.softcap = p->softcap;
+	a.cap_k1 = p->softcap > 0.f ? p->scale / p->softcap : 0.f;
 	a.drop_k0 = (uint32_t)(p->seed & 0xFFFFFFFFull);
 	a.drop_k1 = (uint32_t)(p->seed >> 32);
 	a.seed_dev = (const uint32_t*)p->seed_dev;  // little-endian: low word first
@@ -231,7 +234,7 @@ int fa2_fwd(const fa2_params* p, void* hip_stream) {
 	KArgs a;
 	fill(p, a);
 	// optional scratch: with enough of it a short query over many keys runs split over key ranges
-	size_t need = p->has_window ? 0 : fa2_fwd_scratch_bytes(p);  // (the split forward knows no window)
+	size_t need = (p->has_window || p->softcap > 0.f) ? 0 : fa2_fwd_scratch_bytes(p);  // (the split forward knows no window or soft-capping)
 	if (need && p->scratch && ((uintptr_t)p->scratch & 255) == 0 && p->scratch_bytes >= need) {
 		a.nsplit = fwd_split_plan(p, &a.split_len);
 		a.pack_gqa = fwd_pack_gqa(p) ? 1 : 0;
@@ -239,7 +242,7 @@ int fa2_fwd(const fa2_params* p, void* hip_stream) {
 		a.o_part = (float*)p->scratch;
 		a.lse_part = a.o_part + rows * (size_t)p->D;
 	}
-	hipError_t e = fa2::launch_fwd(p->dtype, p->D, p->bias != nullptr, p->p_drop > 0.f, a, (hipStream_t)hip_stream);
+	hipError_t e = fa2::launch_fwd(p->dtype, p->D, p->bias != nullptr || p->softcap > 0.f, p->p_drop > 0.f, a, (hipStream_t)hip_stream);
 	return e == hipSuccess ? FA2_OK : FA2_EHIP;
 }
 
@@ -254,7 +257,7 @@ static int bwd_launch(const fa2_params* p, void* hip_stream, int stages, void* s
 	a.dk = conv(p->dk);
 	a.dv = conv(p->dv);
 	a.delta = (float*)scratch_ptr;
-	hipError_t e = fa2::launch_bwd(p->dtype, p->D, p->bias != nullptr, p->p_drop > 0.f, a, (hipStream_t)hip_stream);
+	hipError_t e = fa2::launch_bwd(p->dtype, p->D, p->bias != nullptr || p->softcap > 0.f, p->p_drop > 0.f, a, (hipStream_t)hip_stream);
 	return e == hipSuccess ? FA2_OK : FA2_EHIP;
 }
 

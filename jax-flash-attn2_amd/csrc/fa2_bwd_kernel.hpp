@@ -57,8 +57,10 @@ __global__ __launch_bounds__(256) void bwd_delta_kernel(const KArgs a) {
 // dK / dV
 // ---------------------------------------------------------------------------
 // BIAS_T: the bias has the element type of q / k / v (no run-time type dispatch per value)
-template <typename T, int D, int NW, int QB, bool BIAS, bool DROP, bool BIAS_T>
+// CAP: tanh soft-capping of the scores (see the forward kernel); the bias itself may then be absent
+template <typename T, int D, int NW, int QB, bool BIAS, bool DROP, bool BIAS_T, bool CAP = false>
 __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
+	static_assert(!CAP || (BIAS && !BIAS_T), "soft-capping runs on the plain path with bias");
 	typedef typename T::V8 V8;
 	constexpr int BN = NW * 32;     // keys per workgroup
 	constexpr int BMQ = QB * 32;    // query rows per streamed tile
@@ -341,7 +343,9 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 				int row = m0 + 32 * qb + 8 * (i >> 2) + 4 * g + (i & 3);
 				row = row < a.Sq ? row : a.Sq - 1;
 				const char* pp = bias_base + (int64_t)row * a.bias_sm;
-				if constexpr (BIAS_T)
+				if (CAP && a.bias == nullptr)
+					bv[qb & 1][i] = 0.f;
+				else if constexpr (BIAS_T)
 					bv[qb & 1][i] = (float)*(const typename T::E*)pp;
 				else
 					bv[qb & 1][i] = a.bias_dtype == 3   ? *(const float*)pp
@@ -417,6 +421,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		// after it was issued (back-to-back dependent vector operations would each wait for
 		// the previous one's full pipeline latency).
 		float bx[4][4], by[4][4];
+		float bt[4][4];  // CAP: tanh of the scaled score, for the factor 1 - tanh^2 of its derivative
 		// dropout keep bits of a quad (bit e = value 4q + e), produced one value per slot while
 		// the previous quad is processed: one Philox call at a time keeps its registers few
 		uint32_t keepw[4] = {0u, 0u, 0u, 0u};
@@ -491,6 +496,9 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 						if constexpr (BIAS_LDS) {
 							float bvl = (float)__builtin_bit_cast(typename T::V4, bvr[qb & 1][q])[e];
 							bx[q][e] = (__builtin_fmaf(sa[i], c1, bvl) - lse4[q][e]) * kLog2e;
+						} else if constexpr (CAP) {
+							bt[q][e] = tanh_fast(sa[i] * a.cap_k1);
+							bx[q][e] = (__builtin_fmaf(bt[q][e], a.softcap, bv[qb & 1][i]) - lse4[q][e]) * kLog2e;
 						} else {
 							bx[q][e] = (__builtin_fmaf(sa[i], c1, bv[qb & 1][i]) - lse4[q][e]) * kLog2e;
 						}
@@ -519,7 +527,10 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 				}
 			} else if (phase == 2) {
 #pragma unroll
-				for (int e = e0; e < e1; ++e) by[q][e] = __builtin_fabsf(bx[q][e]) * by[q][e];
+				for (int e = e0; e < e1; ++e) {
+					by[q][e] = __builtin_fabsf(bx[q][e]) * by[q][e];
+					if constexpr (CAP) by[q][e] *= __builtin_fmaf(-bt[q][e], bt[q][e], 1.f);
+				}
 			} else {
 				int hf = q >> 1, m = (q & 1) * 2;
 #pragma unroll
@@ -748,8 +759,9 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 // dQ
 // ---------------------------------------------------------------------------
 // BLDS: the bias goes through LDS as in the forward kernel (conditions checked by the launcher)
-template <typename T, int D, int NW, int QB, int WPS, bool BIAS, bool DROP, bool BLDS = false>
+template <typename T, int D, int NW, int QB, int WPS, bool BIAS, bool DROP, bool BLDS = false, bool CAP = false>
 __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
+	static_assert(!CAP || (BIAS && !BLDS), "soft-capping runs on the plain path with bias");
 	typedef typename T::V8 V8;
 	constexpr int BM = NW * QB * 32;
 	constexpr int BN = kFwdBN;
@@ -976,8 +988,12 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 					int i = qrow[qb] < a.Sq ? qrow[qb] : a.Sq - 1;
 					const char* rowp = bias_base + (int64_t)i * a.bias_sm;
 #pragma unroll
-					for (int aa = 0; aa < 4; ++aa)
-						bv[qb][aa] = load_bias4(rowp, n0 + 32 * kb + 8 * aa + 4 * g, a.bias_dtype, a.bias_vec4, a.Sk, a.mask_fill);
+					for (int aa = 0; aa < 4; ++aa) {
+						if (CAP && a.bias == nullptr)
+							bv[qb][aa] = f32x4{0.f, 0.f, 0.f, 0.f};
+						else
+							bv[qb][aa] = load_bias4(rowp, n0 + 32 * kb + 8 * aa + 4 * g, a.bias_dtype, a.bias_vec4, a.Sk, a.mask_fill);
+					}
 				}
 			}
 			f32x16 s[QB], dp[QB];
@@ -1030,8 +1046,11 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 #pragma unroll
 					for (int e = 0; e < 4; ++e) {
 						int i = 4 * aa + e;
-						float p;
-						if constexpr (BIAS)
+						float p, th = 0.f;
+						if constexpr (CAP) {
+							th = tanh_fast(s[qb][i] * a.cap_k1);
+							p = exp2_fast((__builtin_fmaf(th, a.softcap, bv[qb][aa][e]) - lse_r[qb]) * kLog2e);
+						} else if constexpr (BIAS)
 							p = exp2_fast((__builtin_fmaf(s[qb][i], c1, BIAS_LDS ? (float)bvl[aa][e] : bv[qb][aa][e]) - lse_r[qb]) * kLog2e);
 						else
 							p = exp2_fast(__builtin_fmaf(s[qb][i], c1, -lse_r[qb]));
@@ -1042,6 +1061,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 						float dpe = dp[qb][i];
 						if constexpr (DROP) dpe = rnd[e] >= a.drop_thr ? dpe * a.drop_inv_keep : 0.f;
 						s[qb][i] = FOLD_DP ? p * dpe : p * (dpe - del_r[qb]);
+						if constexpr (CAP) s[qb][i] *= __builtin_fmaf(-th, th, 1.f);  // d tanh
 					}
 				}
 #pragma unroll
@@ -1157,7 +1177,9 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 	auto launch_dq = [&]() {
 		a.mtiles = (a.Sq + C::DQ_BM - 1) / C::DQ_BM;
 		dim3 grid((unsigned)(a.mtiles * a.B * a.Hq)), block(C::DQ_NW * 64);
-		if (BIAS && a.bias_lds && D <= 128)
+		if (BIAS && a.softcap > 0.f)
+			hipLaunchKernelGGL((bwd_dq_kernel<T, D, C::DQ_NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, false, BIAS>), grid, block, 0, s, a);
+		else if (BIAS && a.bias_lds && D <= 128)
 			hipLaunchKernelGGL((bwd_dq_kernel<T, D, C::DQ_NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, BIAS>), grid, block, 0, s, a);
 		else
 			hipLaunchKernelGGL((bwd_dq_kernel<T, D, C::DQ_NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, false>), grid, block, 0, s, a);
@@ -1172,7 +1194,9 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 		if (D <= 128 && !a.bias_lds) typed = false;
 		// with bias at D = 128 the streamed tiles are 64 rows, which leaves LDS room for the bias tiles
 		constexpr int QBV = (BIAS && D == 128) ? 2 : C::KV_QB;
-		if (typed)
+		if (BIAS && a.softcap > 0.f)
+			hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, C::KV_NW, QBV, BIAS, DROP, false, BIAS>), grid, block, 0, s, a);
+		else if (typed)
 			hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, C::KV_NW, QBV, BIAS, DROP, BIAS>), grid, block, 0, s, a);
 		else
 			hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, C::KV_NW, QBV, BIAS, DROP, false>), grid, block, 0, s, a);

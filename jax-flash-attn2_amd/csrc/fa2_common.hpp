@@ -108,6 +108,11 @@ FA2_DEV typename T::V8 pack8(float x0, float x1, float x2, float x3, float x4, f
 
 FA2_DEV float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
 FA2_DEV float log2_fast(float x) { return __builtin_amdgcn_logf(x); }
+// tanh(x) = 1 - 2 / (1 + e^(2x)): one exp2, one reciprocal; exactly +-1 at the ends of the range
+FA2_DEV float tanh_fast(float x) {
+	float t = exp2_fast(x * (2.f * kLog2e));
+	return __builtin_fmaf(-2.f, __builtin_amdgcn_rcpf(t + 1.f), 1.f);
+}
 
 // max of the values held by lane l and lane l^32
 FA2_DEV float pair_max(float x) {

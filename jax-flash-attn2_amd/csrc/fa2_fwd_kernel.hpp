@@ -108,8 +108,10 @@ FA2_DEV f32x4 load_bias4(const char* rowp, int col, int dtype, bool vec_ok, int 
 // leave most of the chip idle.
 // BLDS: the bias goes through LDS (the launcher has checked element type, alignment and the key
 // count); otherwise every lane loads its bias values from global memory.
-template <typename T, int D, int NW, int QB, int WPS, bool BIAS, bool DROP, bool SPLIT = false, bool BLDS = false>
+// CAP: tanh soft-capping of the scores (refrence_call.py:48-51), on the path with bias; the bias itself may be absent.
+template <typename T, int D, int NW, int QB, int WPS, bool BIAS, bool DROP, bool SPLIT = false, bool BLDS = false, bool CAP = false>
 __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
+	static_assert(!CAP || (BIAS && !BLDS && !SPLIT), "soft-capping runs on the plain path with bias");
 	typedef typename T::V8 V8;
 	constexpr int BM = NW * QB * 32;
 	constexpr int BN = kFwdBN;
@@ -376,8 +378,12 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 #pragma unroll
 				for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-					for (int aa = 0; aa < 4; ++aa)
-						bv[kb][qb][aa] = load_bias4(rowp, n0 + 32 * kb + 8 * aa + 4 * g, a.bias_dtype, a.bias_vec4, a.Sk, a.mask_fill);
+					for (int aa = 0; aa < 4; ++aa) {
+						if (CAP && a.bias == nullptr)
+							bv[kb][qb][aa] = f32x4{0.f, 0.f, 0.f, 0.f};
+						else
+							bv[kb][qb][aa] = load_bias4(rowp, n0 + 32 * kb + 8 * aa + 4 * g, a.bias_dtype, a.bias_vec4, a.Sk, a.mask_fill);
+					}
 			}
 		}
 
@@ -554,7 +560,11 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 				for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
 					for (int i = 0; i < 16; ++i) {
-						float x = __builtin_fmaf(s[kb][qb][i], c1, bv[kb][qb][i >> 2][i & 3]);
+						float x;
+						if constexpr (CAP)
+							x = __builtin_fmaf(tanh_fast(s[kb][qb][i] * a.cap_k1), a.softcap, bv[kb][qb][i >> 2][i & 3]);
+						else
+							x = __builtin_fmaf(s[kb][qb][i], c1, bv[kb][qb][i >> 2][i & 3]);
 						if constexpr (MASKED) {
 							int j = n0 + 32 * kb + 8 * (i >> 2) + 4 * g + (i & 3);
 							x = (j <= jmax[qb] && j >= jmin[qb]) ? x : -INFINITY;
@@ -805,7 +815,11 @@ hipError_t launch_fwd_t(bool bias, bool drop, KArgs& a, hipStream_t s) {
 	if (bias && a.bias_sh == 0 && a.B % 8 == 0) a.xcd_remap = 2;
 	dim3 grid((unsigned)(a.mtiles * a.B * a.Hq)), block(C::NW * 64);
 	const bool blds = bias && a.bias_lds && D <= 128;
-	if (blds && drop)
+	if (a.softcap > 0.f && drop)
+		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, C::WPS, true, true, false, false, true>), grid, block, 0, s, a);
+	else if (a.softcap > 0.f)
+		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, C::WPS, true, false, false, false, true>), grid, block, 0, s, a);
+	else if (blds && drop)
 		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, C::WPS, true, true, false, true>), grid, block, 0, s, a);
 	else if (blds)
 		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, C::WPS, true, false, false, true>), grid, block, 0, s, a);

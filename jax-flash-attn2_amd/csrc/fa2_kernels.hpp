@@ -29,6 +29,8 @@ struct KArgs {
 	int causal;      // (host side only: the kernels read win_right)
 	int win_left, win_right;  // row i sees keys i + off - win_left .. i + off + win_right; a negative bound is none; causal = win_right 0
 	float scale;
+	float softcap;   // > 0: scores become softcap * tanh(scale * q.k / softcap) before bias and mask (kernel variants CAP)
+	float cap_k1;    // scale / softcap
 	uint32_t drop_k0, drop_k1, drop_thr;
 	const uint32_t* seed_dev;  // when set: the Philox key (low word, high word) is read from device memory instead
 

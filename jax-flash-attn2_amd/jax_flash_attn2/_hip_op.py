@@ -67,7 +67,7 @@ def _usable(x: torch.Tensor) -> torch.Tensor:
 	return x
 
 
-def _fill_common(p, q, k, v, bias, seqlens, scale, p_drop, causal, seed, kv_lens=None, window=None):
+def _fill_common(p, q, k, v, bias, seqlens, scale, p_drop, causal, seed, kv_lens=None, window=None, softcap=0.0):
 	B, Sq, Hq, D = q.shape
 	Sk, Hkv = k.shape[1], k.shape[2]
 	p.dtype = _DTYPES[q.dtype]
@@ -92,6 +92,7 @@ def _fill_common(p, q, k, v, bias, seqlens, scale, p_drop, causal, seed, kv_lens
 	if window is not None:
 		left, right = window
 		p.has_window, p.window_left, p.window_right = 1, int(left), int(right)
+	p.softcap = float(softcap or 0.0)
 	if kv_lens is not None:
 		if kv_lens.dtype != torch.int32 or kv_lens.numel() != B or not kv_lens.is_contiguous():
 			raise ValueError("kv_lens must be a contiguous int32 tensor with one entry per batch row")
@@ -146,7 +147,7 @@ def _seqlens_from_mask(attention_mask, q):
 
 
 def fwd(q, k, v, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, causal=False, dropout_seed=None, kv_lens=None,
-        window=None):
+        window=None, softcap=0.0):
 	"""Returns (out [B,Sq,Hq,D] in q.dtype, lse [B,Hq,Sq] fp32 natural log)."""
 	lib = _lib.load()
 	D0 = q.shape[-1]
@@ -158,7 +159,7 @@ def fwd(q, k, v, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, 
 	out = torch.empty((B, Sq, Hq, D), dtype=q.dtype, device=q.device)
 	lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
 	p = _lib.new_params()
-	_fill_common(p, q, k, v, bias, seqlens, scale, dropout_prob, causal, dropout_seed, kv_lens, window)
+	_fill_common(p, q, k, v, bias, seqlens, scale, dropout_prob, causal, dropout_seed, kv_lens, window, softcap)
 	p.o = _t4(out)
 	p.lse = lse.data_ptr()
 	# short query over many keys: scratch lets the library split the keys over workgroups
@@ -172,7 +173,7 @@ def fwd(q, k, v, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, 
 
 
 def bwd(q, k, v, out, lse, dout, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, causal=False,
-        dropout_seed=None, kv_lens=None, window=None):
+        dropout_seed=None, kv_lens=None, window=None, softcap=0.0):
 	"""Returns (dq, dk, dv) in the dtypes of q, k, v; dk/dv summed over each KV group."""
 	lib = _lib.load()
 	D0 = q.shape[-1]
@@ -185,7 +186,7 @@ def bwd(q, k, v, out, lse, dout, bias=None, seqlens=None, softmax_scale=None, dr
 	dk = torch.empty_like(k, memory_format=torch.contiguous_format)
 	dv = torch.empty_like(v, memory_format=torch.contiguous_format)
 	p = _lib.new_params()
-	_fill_common(p, q, k, v, bias, seqlens, scale, dropout_prob, causal, dropout_seed, kv_lens, window)
+	_fill_common(p, q, k, v, bias, seqlens, scale, dropout_prob, causal, dropout_seed, kv_lens, window, softcap)
 	p.o = _t4(out)
 	p.lse = lse.data_ptr()
 	p.dout, p.dq, p.dk, p.dv = _t4(dout), _t4(dq), _t4(dk), _t4(dv)
@@ -217,7 +218,7 @@ class Plan:
 	enqueue kernels, nothing is allocated per call."""
 
 	def __init__(self, q, k, v, dout=None, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, causal=False,
-	             dropout_seed=None, kv_lens=None, window=None):
+	             dropout_seed=None, kv_lens=None, window=None, softcap=0.0):
 		self.lib = _lib.load()
 		self.q, self.k, self.v = _usable(q), _usable(k), _usable(v)
 		self.bias = _prep_bias(bias)
@@ -228,7 +229,7 @@ class Plan:
 		self.lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
 		p = self.params = _lib.new_params()
 		self.kv_lens = kv_lens
-		_fill_common(p, self.q, self.k, self.v, self.bias, seqlens, scale, dropout_prob, causal, dropout_seed, kv_lens, window)
+		_fill_common(p, self.q, self.k, self.v, self.bias, seqlens, scale, dropout_prob, causal, dropout_seed, kv_lens, window, softcap)
 		self.seed = dropout_seed  # (a device-resident seed must outlive the plan's calls)
 		p.o = _t4(self.out)
 		p.lse = self.lse.data_ptr()
@@ -265,18 +266,18 @@ class _FlashAttentionFn(torch.autograd.Function):
 	(_flash_attention.py:119-122).  Returns (dq, dk, dv) and None for everything else."""
 
 	@staticmethod
-	def forward(ctx, q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens=None, window=None):
-		out, lse = fwd(q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens, window)
+	def forward(ctx, q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens=None, window=None, softcap=0.0):
+		out, lse = fwd(q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens, window, softcap)
 		ctx.save_for_backward(q, k, v, bias, seqlens, out, lse, kv_lens)
-		ctx.cfg = (softmax_scale, dropout_prob, causal, dropout_seed, window)
+		ctx.cfg = (softmax_scale, dropout_prob, causal, dropout_seed, window, softcap)
 		return out
 
 	@staticmethod
 	def backward(ctx, dout):
 		q, k, v, bias, seqlens, out, lse, kv_lens = ctx.saved_tensors
-		softmax_scale, dropout_prob, causal, dropout_seed, window = ctx.cfg
-		dq, dk, dv = bwd(q, k, v, out, lse, dout, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens, window)
-		return dq, dk, dv, None, None, None, None, None, None, None, None
+		softmax_scale, dropout_prob, causal, dropout_seed, window, softcap = ctx.cfg
+		dq, dk, dv = bwd(q, k, v, out, lse, dout, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens, window, softcap)
+		return dq, dk, dv, None, None, None, None, None, None, None, None, None
 
 
 def flash_attention(
@@ -293,6 +294,7 @@ def flash_attention(
 	*,
 	kv_lens=None,
 	window_size=None,
+	softcap: float = 0.0,
 ):
 	"""Same signature as the reference's `triton_flash_attention`
 	(_flash_attention.py:125-157).  `varlen_mode` is accepted for source
@@ -301,11 +303,13 @@ def flash_attention(
 	int32 [B] number of valid keys per batch row - key padding that may be combined
 	with a bias and with Sq != Sk, which the 2-D attention_mask may not.  `window_size` =
 	(left, right) (keyword only): the sliding window of the reference's naive attention
-	(refrence_call.py:32,55-75); a negative bound is none, causal sets right = 0."""
+	(refrence_call.py:32,55-75); a negative bound is none, causal sets right = 0.  `softcap` > 0
+	(keyword only): scores become softcap * tanh(score / softcap) before bias and masks
+	(refrence_call.py:33,48-51)."""
 	del varlen_mode
 	if attention_mask is not None and attention_mask.dim() == 4:
 		assert bias is None, "Attention mask is not supported along with attention bias. Just use bias instead."
 		bias, attention_mask = _mask_operand(attention_mask, q), None
 	check_shapes(q, k, v, bias, attention_mask)
 	seqlens = _seqlens_from_mask(attention_mask, q)
-	return _FlashAttentionFn.apply(q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens, window_size)
+	return _FlashAttentionFn.apply(q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens, window_size, softcap)

@@ -62,6 +62,7 @@ class Fa2Params(ctypes.Structure):
 		("has_window", ctypes.c_int32),
 		("window_left", ctypes.c_int32),
 		("window_right", ctypes.c_int32),
+		("softcap", ctypes.c_float),
 	]
 
 

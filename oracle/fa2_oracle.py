@@ -178,7 +178,7 @@ def _ptx(p, x):
 	return np.swapaxes(np.matmul(np.swapaxes(p, 2, 3), _bh(x)), 1, 2)
 
 
-def _scores(q, k, bias, scale, causal, seqlens, dtype, kv_lens=None, window=None):
+def _scores(q, k, bias, scale, causal, seqlens, dtype, kv_lens=None, window=None, softcap=0.0, return_tanh=False):
 	B, Sq, Hq, D = q.shape
 	_, Sk, Hkv, _ = k.shape
 	if Hq % Hkv:
@@ -187,16 +187,23 @@ def _scores(q, k, bias, scale, causal, seqlens, dtype, kv_lens=None, window=None
 	qf = np.asarray(q, dtype=dtype)
 	kf = np.repeat(np.asarray(k, dtype=dtype), r, axis=2)  # q-head h uses kv-head h // r
 	s = _qk(qf, kf) * dtype(scale)
+	th = None
+	if softcap and softcap > 0:
+		# tanh soft-capping of the scaled scores, before masks and bias (refrence_call.py:48-51)
+		th = np.tanh(s / dtype(softcap))
+		s = th * dtype(softcap)
 	bb = _expand_bias(bias, B, Hq, Hkv, Sq, Sk, dtype)
 	if bb is not None:
 		s = s + bb
 	ok = allowed_mask(B, Sq, Sk, causal, seqlens, kv_lens, window)[:, None]
 	s = np.where(ok, s, -np.inf)
+	if return_tanh:
+		return s, ok, r, th
 	return s, ok, r
 
 
 def attention_fwd(q, k, v, bias=None, causal=False, scale=None, seqlens=None,
-                  p_drop=0.0, seed=0, dtype=np.float64, return_probs=False, pos_offset=(0, 0, 0), kv_lens=None, window=None):
+                  p_drop=0.0, seed=0, dtype=np.float64, return_probs=False, pos_offset=(0, 0, 0), kv_lens=None, window=None, softcap=0.0):
 	"""O [B,Sq,Hq,D] and LSE [B,Hq,Sq] (natural log) of exact attention.
 
 	q [B,Sq,Hq,D], k/v [B,Sk,Hkv,D].  Rows with no allowed key give O = 0 and
@@ -206,7 +213,7 @@ def attention_fwd(q, k, v, bias=None, causal=False, scale=None, seqlens=None,
 	B, Sq, Hq, D = q.shape
 	Sk, Hkv = k.shape[1], k.shape[2]
 	scale = (1.0 / math.sqrt(D)) if scale is None else scale
-	s, ok, r = _scores(q, k, bias, scale, causal, seqlens, dtype, kv_lens, window)
+	s, ok, r = _scores(q, k, bias, scale, causal, seqlens, dtype, kv_lens, window, softcap)
 	m = np.max(s, axis=-1, keepdims=True)
 	m_safe = np.where(np.isfinite(m), m, 0.0)
 	e = np.exp(s - m_safe)
@@ -226,7 +233,7 @@ def attention_fwd(q, k, v, bias=None, causal=False, scale=None, seqlens=None,
 
 
 def attention_bwd(q, k, v, dO, bias=None, causal=False, scale=None, seqlens=None,
-                  p_drop=0.0, seed=0, dtype=np.float64, pos_offset=(0, 0, 0), kv_lens=None, window=None):
+                  p_drop=0.0, seed=0, dtype=np.float64, pos_offset=(0, 0, 0), kv_lens=None, window=None, softcap=0.0):
 	"""Analytic gradients (dQ, dK, dV) of sum(O * dO); FlashAttention-2 Algorithm 2,
 	the same five products as flash_attention_jax/_backward_jax.py:111-127, with
 	dK/dV summed over the q-heads of each KV group (_backward_triton.py:1156-1161).
@@ -234,7 +241,7 @@ def attention_bwd(q, k, v, dO, bias=None, causal=False, scale=None, seqlens=None
 	B, Sq, Hq, D = q.shape
 	Sk, Hkv = k.shape[1], k.shape[2]
 	scale = (1.0 / math.sqrt(D)) if scale is None else scale
-	o, lse, p, pd = attention_fwd(q, k, v, bias, causal, scale, seqlens, p_drop, seed, dtype, True, pos_offset, kv_lens, window)
+	o, lse, p, pd = attention_fwd(q, k, v, bias, causal, scale, seqlens, p_drop, seed, dtype, True, pos_offset, kv_lens, window, softcap)
 	r = Hq // Hkv
 	dOf = np.asarray(dO, dtype=dtype)
 	qf = np.asarray(q, dtype=dtype)
@@ -249,6 +256,10 @@ def attention_bwd(q, k, v, dO, bias=None, causal=False, scale=None, seqlens=None
 		dp = dpd
 	delta = np.einsum("bihd,bihd->bhi", o, dOf)[..., None]  # = rowsum(P * dP)
 	ds = p * (dp - delta)
+	if softcap and softcap > 0:
+		# d/dx [c tanh(x / c)] = 1 - tanh^2(x / c)
+		th = _scores(q, k, None, scale, False, None, dtype, softcap=softcap, return_tanh=True)[3]
+		ds = ds * (1.0 - th * th)
 	dq = _pv(ds, kf) * dtype(scale)
 	dk_full = _ptx(ds, qf) * dtype(scale)
 	dk = dk_full.reshape(B, Sk, Hkv, r, D).sum(axis=3)

@@ -1,6 +1,7 @@
 """Pins the CPU oracle: known-answer vectors, closed forms, invariants, finite
 differences and the committed golden fixtures.  No GPU."""
 
+import math
 import os
 
 import numpy as np
@@ -133,7 +134,8 @@ def test_bias_broadcast_rules():
 @pytest.mark.parametrize(
 	"kw",
 	[dict(), dict(causal=True), dict(bias=True), dict(causal=True, p_drop=0.3, seed=7), dict(seqlens=[5, 6]),
-	 dict(causal=True, scale=0.7)],
+	 dict(causal=True, scale=0.7), dict(softcap=0.8), dict(causal=True, bias=True, softcap=1.5, p_drop=0.2, seed=3),
+	 dict(window=(2, 1), kv_lens=[6, 4])],
 )
 def test_backward_matches_finite_differences(kw):
 	rng = np.random.default_rng(5)
@@ -224,6 +226,29 @@ def test_sliding_window_is_the_local_mask_of_the_naive_reference():
 		assert np.allclose(a, b)
 	o, lse = O.attention_fwd(q[:, :, :, :], k[:, :3], v[:, :3], window=(1, 0))  # Sq 9 > Sk 3: the first rows see nothing
 	assert np.all(o[:, :5] == 0) and np.all(np.isneginf(lse[..., :5]))
+
+
+def test_softcap_is_the_tanh_capping_of_the_naive_reference():
+	"""refrence_call.py:48-51: scores / softcap -> tanh -> * softcap, on the scaled scores, before masks and bias.
+	Against scipy's softmax of the formula written out; a large cap changes nothing; scores stay within +-cap."""
+	rng = np.random.default_rng(11)
+	B, Sq, Sk, Hq, Hkv, D = 2, 7, 9, 4, 2, 8
+	q, k, v, _ = _rand(rng, B, Sq, Sk, Hq, Hkv, D)
+	q = q * 3.0
+	bias = rng.normal(size=(B, Hq, Sq, Sk))
+	cap = 1.3
+	kr = np.repeat(k, 2, axis=2)
+	vr = np.repeat(v, 2, axis=2)
+	sc = np.einsum("bthd,bshd->bhts", q / math.sqrt(D), kr)
+	assert np.abs(sc).max() > 2 * cap  # the cap bites
+	x = np.tanh(sc / cap) * cap + bias
+	want = np.einsum("bhts,bshd->bthd", scipy.special.softmax(x, axis=-1), vr)
+	o, lse = O.attention_fwd(q, k, v, bias=bias, softcap=cap)
+	assert np.allclose(o, want)
+	assert np.allclose(lse, scipy.special.logsumexp(x, axis=-1))
+	o_big, _ = O.attention_fwd(q, k, v, bias=bias, softcap=1e9)
+	o_off, _ = O.attention_fwd(q, k, v, bias=bias)
+	assert np.allclose(o_big, o_off, atol=1e-9)
 
 
 def test_blockwise_restatement_equals_closed_form():

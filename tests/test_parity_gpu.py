@@ -340,6 +340,50 @@ def test_sliding_window(window):
 	check_grads((qq.grad,), (g_ref[0],), f"window {window} with key lengths")
 
 
+@pytest.mark.parametrize("cap", [1.0, 5.0, 30.0])
+def test_softcap(cap):
+	"""tanh soft-capping of the scores (refrence_call.py:33,48-51), fused: forward and backward against the oracle with
+	scores that reach several times the cap (so that tanh saturates) and scores well inside it; with and without
+	bias (all element types, the mask bytes too), causal, GQA, every head dim, dropout, key lengths, a window and a
+	short query (which otherwise takes the split forward)."""
+	cases = (
+		# B, Sq, Sk, Hq, Hkv, D, dtype, causal, bias shape, bias dtype, p, qk_scale
+		(2, 320, 320, 4, 2, 128, torch.bfloat16, True, None, None, 0.0, 2.1),
+		(1, 200, 333, 4, 4, 64, torch.float16, False, None, None, 0.0, 2.1),
+		(1, 160, 160, 2, 1, 256, torch.bfloat16, True, None, None, 0.0, 1.0),
+		(2, 160, 224, 4, 2, 64, torch.bfloat16, False, (2, 1, 160, 224), None, 0.0, 2.1),
+		(2, 160, 224, 4, 2, 128, torch.bfloat16, True, (1, 4, 160, 224), torch.float32, 0.0, 1.0),
+		(1, 192, 192, 4, 2, 128, torch.bfloat16, True, None, None, 0.2, 2.1),
+		(1, 130, 130, 2, 2, 256, torch.float16, False, (1, 2, 130, 130), None, 0.1, 1.0),
+		(2, 16, 1024, 4, 2, 128, torch.bfloat16, False, None, None, 0.0, 2.1),
+	)
+	for (B, Sq, Sk, Hq, Hkv, D, dtype, causal, bshape, bdt, p, qs) in cases:
+		q, k, v, do, bias = make_inputs(B, Sq, Sk, Hq, Hkv, D, dtype, 61, bshape, bias_dtype=bdt, qk_scale=qs)
+		kw = dict(causal=causal, p_drop=p, seed=4, softcap=cap)
+		o_ref, lse_ref = O.attention_fwd(f64(q), f64(k), f64(v), f64(bias), **kw)
+		g_ref = O.attention_bwd(f64(q), f64(k), f64(v), f64(do), f64(bias), **kw)
+		o, lse = op.fwd(_dev(q), _dev(k), _dev(v), _dev(bias), None, None, p, causal, 4, softcap=cap)
+		gr = op.bwd(_dev(q), _dev(k), _dev(v), o, lse, _dev(do), _dev(bias), None, None, p, causal, 4, softcap=cap)
+		what = f"softcap {cap} B{B} Sq{Sq} Sk{Sk} Hq{Hq} Hkv{Hkv} D{D} {dtype} causal={causal} bias={bshape} {bdt} p={p}"
+		check_forward(o, lse, o_ref, lse_ref, dtype, what)
+		check_grads(gr, g_ref, what)
+	# with a boolean mask operand, key lengths and a window, through the differentiation rule
+	q, k, v, do, _ = make_inputs(2, 150, 150, 2, 2, 64, torch.bfloat16, 62, qk_scale=2.1)
+	kl = torch.tensor([150, 90], dtype=torch.int32, device=DEV)
+	qq, kk, vv = (_dev(x).requires_grad_() for x in (q, k, v))
+	out = op.flash_attention(qq, kk, vv, kv_lens=kl, window_size=(40, 3), softcap=cap)
+	out.backward(_dev(do))
+	kw = dict(kv_lens=[150, 90], window=(40, 3), softcap=cap)
+	o_ref, _ = O.attention_fwd(f64(q), f64(k), f64(v), **kw)
+	g_ref = O.attention_bwd(f64(q), f64(k), f64(v), f64(do), **kw)
+	assert np.abs(out.detach().float().cpu().numpy() - o_ref).max() <= TOL_O[torch.bfloat16]
+	check_grads((qq.grad, kk.grad, vv.grad), g_ref, f"softcap {cap} with key lengths and a window")
+	# cap off (0) is the plain operator
+	o0, lse0 = op.fwd(_dev(q), _dev(k), _dev(v), softcap=0.0)
+	o1, lse1 = op.fwd(_dev(q), _dev(k), _dev(v))
+	assert torch.equal(o0, o1) and torch.equal(lse0, lse1)
+
+
 def test_mask_as_finfo_min_bias():
 	"""Boolean mask -> where(mask, 0, finfo.min) bias (the README recipe) must equal key-length masking."""
 	B, S, H, D = 2, 192, 4, 64
