@@ -116,13 +116,19 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		int id = blockIdx.x;
 		int per_group = a.mtiles;
 		int grp, within;
-		if (a.xcd_remap == 2) {
+		if (a.xcd_remap >= 2) {
 			// bias shared by the heads: one batch per XCD, the kv-heads of one key tile adjacent
 			int xcd = id & 7, j = id >> 3;
 			int per_batch = per_group * a.Hkv;
 			int rem = j % per_batch;
 			grp = ((j / per_batch) * 8 + xcd) * a.Hkv + rem % a.Hkv;
 			within = rem / a.Hkv;
+			if (a.xcd_remap == 3) {
+				// batch rows of different key lengths: the units (batch, key tile) of one batch go round the XCDs
+				int u = j / a.Hkv, nb8 = a.B >> 3;
+				within = u / nb8;
+				grp = (((xcd - within) & 7) + 8 * (u % nb8)) * a.Hkv + j % a.Hkv;
+			}
 		} else if (a.xcd_remap) {
 			int xcd = id & 7, j = id >> 3;
 			grp = (j / per_group) * 8 + xcd;
@@ -188,6 +194,11 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		q_hi = e < q_hi ? e : q_hi;
 	}
 	if (n0 >= sk_eff) q_hi = q_lo;
+	// rows that may see this lane's key: row_lo .. row_hi (none when the key itself is beyond the valid ones)
+	int row_lo = wr >= 0 ? jcol - off - wr : -(1 << 30);
+	int row_hi = sq_eff - 1;
+	if (wl >= 0) row_hi = jcol - off + wl < row_hi ? jcol - off + wl : row_hi;
+	if (jcol >= sk_eff) row_lo = 1 << 30;
 	const int nq = q_hi > q_lo ? q_hi - q_lo : 0;
 	const int steps = nq * r;
 
@@ -472,7 +483,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 						float p = exp2_fast(bx[q][e]);
 						if constexpr (MASKED) {
 							int row = m0 + 32 * qb + 8 * q + 4 * g + e;
-							bool ok = row < sq_eff && jcol < sk_eff && (wr < 0 || jcol <= row + off + wr) && (wl < 0 || jcol >= row + off - wl);
+							bool ok = (row >= row_lo) & (row <= row_hi);  // (no short-circuit: that would be a divergent branch per value)
 							p = ok ? p : 0.f;
 						}
 						bx[q][e] = p;
@@ -514,7 +525,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 					float p = exp2_fast(bx[q][e]);
 					int row = m0 + 32 * qb + 8 * q + 4 * g + e;
 					if constexpr (MASKED) {
-						bool ok = row < sq_eff && jcol < sk_eff && (wr < 0 || jcol <= row + off + wr) && (wl < 0 || jcol >= row + off - wl);
+						bool ok = (row >= row_lo) & (row <= row_hi);  // (no short-circuit: that would be a divergent branch per value)
 						p = ok ? p : 0.f;
 					}
 					bx[q][e] = p;
@@ -1056,7 +1067,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 							p = exp2_fast(__builtin_fmaf(s[qb][i], c1, -lse_r[qb]));
 						if constexpr (MASKED) {
 							int j = n0 + 32 * kb + 8 * aa + 4 * g + e;
-							p = (j <= jmax[qb] && j >= jmin[qb]) ? p : 0.f;
+							p = ((j <= jmax[qb]) & (j >= jmin[qb])) ? p : 0.f;
 						}
 						float dpe = dp[qb][i];
 						if constexpr (DROP) dpe = rnd[e] >= a.drop_thr ? dpe * a.drop_inv_keep : 0.f;
@@ -1163,7 +1174,7 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 	typedef BwdCfg<T, D> C;
 	int groups = a.B * a.Hkv;
 	a.xcd_remap = (groups % 8 == 0) ? 1 : 0;
-	if (BIAS && a.bias_sh == 0 && a.B % 8 == 0) a.xcd_remap = 2;
+	if (BIAS && a.bias_sh == 0 && a.B % 8 == 0) a.xcd_remap = a.kv_lens ? 3 : 2;
 	// Delta and dQ both requested (the whole backward, or stages 1 + 4): the dQ kernel forms delta
 	// itself and runs first, the dK/dV kernel reads the delta it left in scratch.  Otherwise each
 	// stage is launched as asked and the dQ / dK/dV kernels read the delta of an earlier pre-pass.

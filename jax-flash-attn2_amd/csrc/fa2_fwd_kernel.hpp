@@ -46,6 +46,18 @@ FA2_DEV void decode_block(const KArgs& a, int& mt, int& h, int& b, int id = (int
 		h = rem % a.Hq;
 		return;
 	}
+	if (a.xcd_remap == 3) {
+		// The same sharing of a head-less bias, for batch rows of different key lengths: the unit (batch, row tile)
+		// with its heads adjacent stays on one XCD, but the units of one batch go round the XCDs (batch b, tile t
+		// on XCD (b + t) % 8), so that a short batch row does not leave its XCD idle.
+		int xcd = id & 7, j = id >> 3;
+		int u = j / a.Hq, nb8 = a.B >> 3;
+		int tile = u / nb8;
+		h = j % a.Hq;
+		mt = a.mtiles - 1 - tile;
+		b = ((xcd - tile) & 7) + 8 * (u % nb8);
+		return;
+	}
 	int r = a.Hq / a.Hkv;
 	int per_group = a.mtiles * r;
 	int grp, within;
@@ -492,7 +504,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 								float p = exp2_fast(pv[e]);
 								if constexpr (MASKED) {
 									int j = n0 + 32 * kb + 8 * (2 * hf + (e >> 2)) + 4 * g + (e & 3);
-									p = (j <= jmax[qb] && j >= jmin[qb]) ? p : 0.f;
+									p = ((j <= jmax[qb]) & (j >= jmin[qb])) ? p : 0.f;
 								}
 								ls4[e & 3] += p;
 								pv[e] = p;
@@ -518,7 +530,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 							float x = s[kb][qb][i];
 							if constexpr (MASKED) {
 								int j = n0 + 32 * kb + 8 * (i >> 2) + 4 * g + (i & 3);
-								x = (j <= jmax[qb] && j >= jmin[qb]) ? x : -INFINITY;
+								x = ((j <= jmax[qb]) & (j >= jmin[qb])) ? x : -INFINITY;
 							}
 							s[kb][qb][i] = x;
 							mx4[i & 3] = __builtin_fmaxf(mx4[i & 3], x);
@@ -567,7 +579,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 							x = __builtin_fmaf(s[kb][qb][i], c1, bv[kb][qb][i >> 2][i & 3]);
 						if constexpr (MASKED) {
 							int j = n0 + 32 * kb + 8 * (i >> 2) + 4 * g + (i & 3);
-							x = (j <= jmax[qb] && j >= jmin[qb]) ? x : -INFINITY;
+							x = ((j <= jmax[qb]) & (j >= jmin[qb])) ? x : -INFINITY;
 						}
 						s[kb][qb][i] = x;
 						mx4[i & 3] = __builtin_fmaxf(mx4[i & 3], x);
@@ -812,7 +824,7 @@ hipError_t launch_fwd_t(bool bias, bool drop, KArgs& a, hipStream_t s) {
 	a.mtiles = (a.Sq + C::BM - 1) / C::BM;
 	int groups = a.B * a.Hkv;
 	a.xcd_remap = (groups % 8 == 0) ? 1 : 0;
-	if (bias && a.bias_sh == 0 && a.B % 8 == 0) a.xcd_remap = 2;
+	if (bias && a.bias_sh == 0 && a.B % 8 == 0) a.xcd_remap = a.kv_lens ? 3 : 2;
 	dim3 grid((unsigned)(a.mtiles * a.B * a.Hq)), block(C::NW * 64);
 	const bool blds = bias && a.bias_lds && D <= 128;
 	if (a.softcap > 0.f && drop)
