@@ -131,8 +131,11 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 			}
 		} else if (a.xcd_remap) {
 			int xcd = id & 7, j = id >> 3;
-			grp = (j / per_group) * 8 + xcd;
-			within = j % per_group;
+			// a.interleave = e groups of an XCD advance together: e adjacent workgroups are the same key tile (see launch_order())
+			int e = a.interleave;
+			int sgi = j / (e * per_group), rem = j % (e * per_group);
+			grp = (sgi * e + rem % e) * 8 + xcd;
+			within = rem / e;
 		} else {
 			grp = id / per_group;
 			within = id % per_group;
@@ -1187,6 +1190,7 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 	}
 	auto launch_dq = [&]() {
 		a.mtiles = (a.Sq + C::DQ_BM - 1) / C::DQ_BM;
+		a.interleave = a.xcd_remap == 1 ? launch_order(a, a.Hq / a.Hkv, groups / 8) : 1;
 		dim3 grid((unsigned)(a.mtiles * a.B * a.Hq)), block(C::DQ_NW * 64);
 		if (BIAS && a.softcap > 0.f)
 			hipLaunchKernelGGL((bwd_dq_kernel<T, D, C::DQ_NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, false, BIAS>), grid, block, 0, s, a);
@@ -1198,6 +1202,7 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 	if (fused_delta) launch_dq();
 	if (a.stages & 2) {
 		a.mtiles = (a.Sk + C::KV_BN - 1) / C::KV_BN;
+		a.interleave = a.xcd_remap == 1 ? launch_order(a, 1, groups / 8) : 1;
 		dim3 grid((unsigned)(a.mtiles * a.B * a.Hkv)), block(C::KV_NW * 64);
 		// typed variant: bias in the element type of q; where it stages the bias through LDS (D <= 128)
 		// it also needs 16-byte aligned rows of whole 16-byte pieces

@@ -38,6 +38,7 @@ struct KArgs {
 	int mtiles;      // number of row tiles of the launched kernel
 	int xcd_remap;   // 1: group-major placement of workgroups on the 8 XCDs
 	                 // 2: batch-major placement, heads of a row tile adjacent (a bias shared by the heads stays in L2)
+	int interleave;  // xcd_remap 1: this many (batch, kv-head) groups of an XCD advance through their tiles together (1, 2 or 4)
 	int stages;      // backward: bit 0 delta, bit 1 dK/dV, bit 2 dQ
 	int dq_makes_delta;  // the dQ kernel computes delta itself (and stores it for the dK/dV kernel)
 	// split forward (0 / 1 = off): key ranges of split_len keys, partial results in scratch
