@@ -264,16 +264,19 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	};
 
 	// per-lane LDS byte offsets (swizzle folded in) of the fragments read in the loop
-	int poff[KS];
+	// (the swizzle touches the low four bits of the chunk index only: chunks 16 and up - head dim 256 - are the same
+	// offsets 256 bytes further on, an immediate of the read instead of more registers)
+	constexpr int KR = KS < 8 ? KS : 8, DR = DB < 4 ? DB : 4;
+	int poff[KR];
 #pragma unroll
-	for (int ks = 0; ks < KS; ++ks) poff[ks] = tile_off<D>(c, 2 * ks + g);
-	int toff[DB][2];
+	for (int ks = 0; ks < KR; ++ks) poff[ks] = tile_off<D>(c, 2 * ks + g);
+	int toff[DR][2];
 	{
 		int i16 = lane & 15;
 		int trow = 4 * g + (i16 >> 2);
 		int tcol = 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
 #pragma unroll
-		for (int db = 0; db < DB; ++db) {
+		for (int db = 0; db < DR; ++db) {
 			int col = 32 * db + tcol;
 			toff[db][0] = tile_off<D>(trow, col >> 3) + ((col & 4) << 1);
 			toff[db][1] = tile_off<D>(trow + 8, col >> 3) + ((col & 4) << 1);
@@ -329,13 +332,13 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		// fragment of product j of A(qb): even j -> Q (S), odd j -> dO (dP), k-step j / 2
 		auto issue_A = [&](int qb, int j) __attribute__((always_inline)) {
 			// (poff carries the buffer; dO lies one tile behind Q)
-			afr[(qb * NSLOT + j) % RING] = *(const FA2_LDS V8*)(lds + poff[j >> 1] + ((j & 1) ? TILE_BYTES : 0) + qb * (32 * D * 2));
+			afr[(qb * NSLOT + j) % RING] = *(const FA2_LDS V8*)(lds + poff[(j >> 1) % KR] + ((j >> 1) / KR) * 256 + ((j & 1) ? TILE_BYTES : 0) + qb * (32 * D * 2));
 		};
 		// fragment of product j of C(qb): half j / (2 DB); inside a half even -> dO^T (dV), odd -> Q^T (dK)
 		auto issue_C = [&](int qb, int j) __attribute__((always_inline)) {
 			int hf = j / (2 * DB), rr = j % (2 * DB), db = rr >> 1;
 			const FA2_LDS char* base = lds + ((rr & 1) ? 0 : TILE_BYTES) + qb * (32 * D * 2);
-			cfr[(qb * NSLOT + j) % RING] = lds_tr_issue_rt<D>(base + toff[db][0], base + toff[db][1], hf);
+			cfr[(qb * NSLOT + j) % RING] = lds_tr_issue_rt<D>(base + toff[db % DR][0] + (db / DR) * 256, base + toff[db % DR][1] + (db / DR) * 256, hf);
 		};
 		// statistics of rows 8 aa + 4 g .. + 3 of block qb
 		auto issue_stat = [&](int qb, int aa) __attribute__((always_inline)) {
@@ -705,9 +708,9 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		}
 		// the other buffers next time
 #pragma unroll
-		for (int ks = 0; ks < KS; ++ks) poff[ks] ^= 2 * TILE_BYTES;
+		for (int ks = 0; ks < KR; ++ks) poff[ks] ^= 2 * TILE_BYTES;
 #pragma unroll
-		for (int db = 0; db < DB; ++db) {
+		for (int db = 0; db < DR; ++db) {
 			toff[db][0] ^= 2 * TILE_BYTES;
 			toff[db][1] ^= 2 * TILE_BYTES;
 		}
@@ -969,16 +972,17 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 
 	// (the offsets carry the buffer - K[1] / V[1] / bias[1] lie a power of two behind K[0] / V[0] / bias[0] -
 	// and are flipped after every tile, so that the reads need no address arithmetic in the loop)
-	int koff[KS];
+	constexpr int KR = KS < 8 ? KS : 8, DR = DB < 4 ? DB : 4;  // (chunks 16 and up: + 256 bytes as an immediate, see the dK/dV kernel)
+	int koff[KR];
 #pragma unroll
-	for (int ks = 0; ks < KS; ++ks) koff[ks] = tile_off<D>(c, 2 * ks + g) + (t_begin & 1) * TILE_BYTES;
-	int toff[DB][2];
+	for (int ks = 0; ks < KR; ++ks) koff[ks] = tile_off<D>(c, 2 * ks + g) + (t_begin & 1) * TILE_BYTES;
+	int toff[DR][2];
 	{
 		int i16 = lane & 15;
 		int trow = 4 * g + (i16 >> 2);
 		int tcol = 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
 #pragma unroll
-		for (int db = 0; db < DB; ++db) {
+		for (int db = 0; db < DR; ++db) {
 			int col = 32 * db + tcol;
 			toff[db][0] = tile_off<D>(trow, col >> 3) + ((col & 4) << 1) + (t_begin & 1) * TILE_BYTES;
 			toff[db][1] = tile_off<D>(trow + 8, col >> 3) + ((col & 4) << 1) + (t_begin & 1) * TILE_BYTES;
@@ -1018,10 +1022,10 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 			__builtin_amdgcn_sched_barrier(0);
 #pragma unroll
 			for (int ks = 0; ks < KS; ++ks) {
-				V8 ka = *(const FA2_LDS V8*)(lds + koff[ks] + kb * (32 * D * 2));
+				V8 ka = *(const FA2_LDS V8*)(lds + koff[ks % KR] + (ks / KR) * 256 + kb * (32 * D * 2));
 #pragma unroll
 				for (int qb = 0; qb < QB; ++qb) s[qb] = mfma32(ka, qf[qb][ks], s[qb]);
-				V8 va = *(const FA2_LDS V8*)(lds + koff[ks] + 2 * TILE_BYTES + kb * (32 * D * 2));
+				V8 va = *(const FA2_LDS V8*)(lds + koff[ks % KR] + (ks / KR) * 256 + 2 * TILE_BYTES + kb * (32 * D * 2));
 #pragma unroll
 				for (int qb = 0; qb < QB; ++qb) dp[qb] = mfma32(va, dof[qb][ks], (FOLD_DP && ks == 0) ? ndel16[qb] : dp[qb]);
 			}
@@ -1043,7 +1047,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 			const FA2_LDS char* kt_a = lds + kb * (32 * D * 2);
 			auto issue_k = [&](int hf, u32x4(&dst)[DB]) {
 #pragma unroll
-				for (int db = 0; db < DB; ++db) dst[db] = lds_tr_issue_rt<D>(kt_a + toff[db][0], kt_a + toff[db][1], hf);
+				for (int db = 0; db < DB; ++db) dst[db] = lds_tr_issue_rt<D>(kt_a + toff[db % DR][0] + (db / DR) * 256, kt_a + toff[db % DR][1] + (db / DR) * 256, hf);
 			};
 			issue_k(0, kfr[0]);
 			if constexpr (BOTH_EARLY) issue_k(1, kfr[1]);
@@ -1119,9 +1123,9 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 		if (!skip) tile_body(masked_tag, n0);
 		// the other buffers next time
 #pragma unroll
-		for (int ks = 0; ks < KS; ++ks) koff[ks] ^= TILE_BYTES;
+		for (int ks = 0; ks < KR; ++ks) koff[ks] ^= TILE_BYTES;
 #pragma unroll
-		for (int db = 0; db < DB; ++db) {
+		for (int db = 0; db < DR; ++db) {
 			toff[db][0] ^= TILE_BYTES;
 			toff[db][1] ^= TILE_BYTES;
 		}

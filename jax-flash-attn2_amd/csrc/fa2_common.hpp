@@ -27,6 +27,15 @@ typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
+// f(integral_constant<int, I>) for I = FROM .. TO - 1, unrolled at compile time
+template <int FROM, int TO, typename F>
+FA2_DEV void static_for(F&& f) {
+	if constexpr (FROM < TO) {
+		f(std::integral_constant<int, FROM>{});
+		static_for<FROM + 1, TO>(f);
+	}
+}
+
 // Element traits: E = storage element, V8/V4/V2 = vectors of it.
 struct BF16 {
 	typedef __bf16 E;
@@ -232,31 +241,46 @@ struct TileLoader {
 	static constexpr int TOTAL = ROWS * CPR;
 	static constexpr int NIT = TOTAL / NTHREADS;  // 64 x 16 byte pieces per wave and tile
 	static_assert(TOTAL % NTHREADS == 0, "tile must divide over the workgroup");
-	uint32_t off[NIT];
+	// Rows of 512 bytes (head dim 256) make eight pieces per tile and registers are short there.  Piece `it`
+	// covers rows it * RPI + tid / CPR, and the swizzle repeats every 16 rows: pieces P apart differ by a
+	// whole number of 16-row blocks, which goes into the wave-uniform base address.  Only the first NP offsets
+	// are kept; a tile that needs clamping (ragged end) computes its offsets as it goes.
+	static constexpr bool COMPACT = D >= 256 && NTHREADS % CPR == 0;
+	static constexpr int RPI = NTHREADS / CPR;
+	static constexpr int P = RPI >= 16 ? 1 : 16 / RPI;
+	static constexpr int NP = COMPACT ? (NIT < P ? NIT : P) : NIT;
+	uint32_t off[NP];
 	int rows_state;  // the offsets clamp rows to [0, rows_state)
 	int cols_state;  // ... and 16-byte chunks of a row to [0, cols_state)
 	int wave_slot;   // byte offset of this wave's 64 x 16 bytes inside a piece (scalar)
 
+	static FA2_DEV uint32_t offset_of(int it, int64_t stride_bytes, int tid, int rows_valid, int chunks_valid) {
+		int slot = it * NTHREADS + tid;
+		int row = slot / CPR;
+		int chunk = (slot % CPR) ^ swz<D>(row);
+		int grow = row < rows_valid ? row : rows_valid - 1;
+		int gchunk = chunk < chunks_valid ? chunk : chunks_valid - 1;
+		return (uint32_t)grow * (uint32_t)stride_bytes + (uint32_t)(gchunk << 4);
+	}
 	// stride_bytes * ROWS must fit 31 bits (the launcher checks)
 	FA2_DEV void init(int64_t stride_bytes, int tid, int rows_valid = ROWS, int chunks_valid = CPR) {
 		rows_state = rows_valid;
 		cols_state = chunks_valid;
 		wave_slot = __builtin_amdgcn_readfirstlane((tid >> 6) << 10);
 #pragma unroll
-		for (int it = 0; it < NIT; ++it) {
-			int slot = it * NTHREADS + tid;
-			int row = slot / CPR;
-			int chunk = (slot % CPR) ^ swz<D>(row);
-			int grow = row < rows_valid ? row : rows_valid - 1;
-			int gchunk = chunk < chunks_valid ? chunk : chunks_valid - 1;
-			off[it] = (uint32_t)grow * (uint32_t)stride_bytes + (uint32_t)(gchunk << 4);
-		}
+		for (int it = 0; it < NP; ++it)
+			off[it] = COMPACT ? offset_of(it, stride_bytes, tid, ROWS, CPR) : offset_of(it, stride_bytes, tid, rows_valid, chunks_valid);
 	}
 	// make the offsets fit a tile with rows_valid rows of chunks_valid chunks (wave-uniform; recomputes only on change)
 	FA2_DEV void fit(int64_t stride_bytes, int tid, int rows_valid, int chunks_valid = CPR) {
 		rows_valid = rows_valid < ROWS ? rows_valid : ROWS;
 		chunks_valid = chunks_valid < CPR ? chunks_valid : CPR;
-		if (rows_valid != rows_state || chunks_valid != cols_state) init(stride_bytes, tid, rows_valid, chunks_valid);
+		if constexpr (COMPACT) {
+			rows_state = rows_valid;
+			cols_state = chunks_valid;
+		} else {
+			if (rows_valid != rows_state || chunks_valid != cols_state) init(stride_bytes, tid, rows_valid, chunks_valid);
+		}
 	}
 	// a wave-uniform pointer as an explicitly scalar value
 	static FA2_DEV const char* uniform(const char* p) {
@@ -273,8 +297,20 @@ struct TileLoader {
 	FA2_DEV void load(FA2_LDS char* tile, const char* gbase, int64_t stride_bytes, int rows_valid, int tid, int chunks_valid = CPR) {
 		fit(stride_bytes, tid, rows_valid, chunks_valid);
 		const char* ub = uniform(gbase);
+		if constexpr (COMPACT) {
+			if (rows_state == ROWS && cols_state == CPR) {
 #pragma unroll
-		for (int it = 0; it < NIT; ++it) load_one(tile, ub, it, tid);
+				for (int it = 0; it < NIT; ++it)
+					lds_dma16_so(off[it % NP], ub + (int64_t)((it / NP) * NP * RPI) * stride_bytes, tile + it * NTHREADS * 16 + wave_slot);
+			} else {
+#pragma unroll
+				for (int it = 0; it < NIT; ++it)
+					lds_dma16_so(offset_of(it, stride_bytes, tid, rows_state, cols_state), ub, tile + it * NTHREADS * 16 + wave_slot);
+			}
+		} else {
+#pragma unroll
+			for (int it = 0; it < NIT; ++it) load_one(tile, ub, it, tid);
+		}
 	}
 };
 

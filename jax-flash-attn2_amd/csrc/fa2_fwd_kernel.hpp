@@ -369,16 +369,19 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 	// The offsets carry the buffer (K[1] / V[1] / bias[1] lie a power of two behind K[0] / V[0] / bias[0])
 	// and are flipped after every tile, so that the reads need no address arithmetic in the loop.
 	const int buf0 = t_begin & 1;
-	int koff[KS];
+	// (the swizzle touches the low four bits of the chunk index only: chunks 16 and up - head dim 256 - are the same
+	// offsets 256 bytes further on, an immediate of the read instead of eight more registers)
+	constexpr int KR = KS < 8 ? KS : 8, DR = DB < 4 ? DB : 4;
+	int koff[KR];
 #pragma unroll
-	for (int ks = 0; ks < KS; ++ks) koff[ks] = tile_off<D>(c, 2 * ks + g) + buf0 * TILE_BYTES;
-	int voff[DB][2];
+	for (int ks = 0; ks < KR; ++ks) koff[ks] = tile_off<D>(c, 2 * ks + g) + buf0 * TILE_BYTES;
+	int voff[DR][2];
 	{
 		int i16 = lane & 15;
 		int vrow = 4 * g + (i16 >> 2);
 		int vcol = 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
 #pragma unroll
-		for (int db = 0; db < DB; ++db) {
+		for (int db = 0; db < DR; ++db) {
 			int col = 32 * db + vcol;
 			voff[db][0] = tile_off<D>(vrow, col >> 3) + ((col & 4) << 1) + (2 + buf0) * TILE_BYTES;
 			voff[db][1] = tile_off<D>(vrow + 8, col >> 3) + ((col & 4) << 1) + (2 + buf0) * TILE_BYTES;
@@ -431,14 +434,14 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 			for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
 				for (int kb = 0; kb < KB; ++kb) {
-					V8 kf = *(const FA2_LDS V8*)(lds + koff[ks] + kb * (32 * D * 2));
+					V8 kf = *(const FA2_LDS V8*)(lds + koff[ks % KR] + (ks / KR) * 256 + kb * (32 * D * 2));
 #pragma unroll
 					for (int qb = 0; qb < QB; ++qb) s[kb][qb] = mfma32(kf, qf[qb][ks], s[kb][qb]);
 				}
 			// issue order: a few fragment reads ahead, then one read per product, so that the
 			// LDS latency is paid once per tile instead of once per product
 			{
-				constexpr int NR = KS * KB, PF = NR < 8 ? NR : 8;
+				constexpr int NR = KS * KB, PF = D == 256 ? 4 : (NR < 8 ? NR : 8);  // (head dim 256: registers are short)
 				__builtin_amdgcn_sched_group_barrier(0x100, PF, 0);
 #pragma unroll
 				for (int i = 0; i < NR - PF; ++i) {
@@ -453,18 +456,17 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 		// V fragments for O^T += V^T P^T, fetched in batches of NF; the first batch is in
 		// flight during the softmax, each further one during the products of the previous.
 		constexpr int KK = BN / 16;
-		constexpr int FPB = (8 / DB) < 1 ? 1 : ((8 / DB) > KK ? KK : (8 / DB));  // 16-key steps per batch
-		constexpr int NBATCH = KK / FPB;
-		constexpr int NF = FPB * DB;
+		constexpr int NFR = KK * DB;                                  // fragments of a tile: 16-key step fi / DB, d-block fi % DB
+		constexpr int NF = D == 256 ? 4 : (NFR < 8 ? NFR : 8);        // fragments per batch (head dim 256: registers are short)
+		constexpr int NBATCH = NFR / NF;
 		u32x4 vfr[2][NF];
 		auto issue_v = [&](auto batch_tag, u32x4(&dst)[NF]) {
 			constexpr int BI = decltype(batch_tag)::value;
 #pragma unroll
-			for (int f = 0; f < FPB; ++f)
-#pragma unroll
-				for (int db = 0; db < DB; ++db) {
-					dst[f * DB + db] = lds_tr_issue_rt<D>(lds + voff[db][0], lds + voff[db][1], BI * FPB + f);
-				}
+			for (int u = 0; u < NF; ++u) {
+				const int fi = BI * NF + u, st = fi / DB, db = fi % DB;
+				dst[u] = lds_tr_issue_rt<D>(lds + voff[db % DR][0] + (db / DR) * 256, lds + voff[db % DR][1] + (db / DR) * 256, st);
+			}
 		};
 
 		// online softmax, one query row per lane
@@ -640,18 +642,14 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 			constexpr int BI = decltype(batch_tag)::value;
 			if constexpr (BI + 1 < NBATCH) issue_v(std::integral_constant<int, BI + 1>{}, vfr[(BI + 1) & 1]);
 #pragma unroll
-			for (int f = 0; f < FPB; ++f)
+			for (int u = 0; u < NF; ++u) {
+				const int fi = BI * NF + u, st = fi / DB, db = fi % DB;
 #pragma unroll
-				for (int db = 0; db < DB; ++db)
-#pragma unroll
-					for (int qb = 0; qb < QB; ++qb)
-						oacc[qb][db] = mfma32(as_frag<T>(vfr[BI & 1][f * DB + db]), pf[qb][BI * FPB + f], oacc[qb][db]);
+				for (int qb = 0; qb < QB; ++qb) oacc[qb][db] = mfma32(as_frag<T>(vfr[BI & 1][u]), pf[qb][st], oacc[qb][db]);
+			}
 		};
 		__builtin_amdgcn_sched_barrier(0);
-		pv_batch(std::integral_constant<int, 0>{});
-		if constexpr (NBATCH > 1) pv_batch(std::integral_constant<int, 1>{});
-		if constexpr (NBATCH > 2) pv_batch(std::integral_constant<int, 2>{});
-		if constexpr (NBATCH > 3) pv_batch(std::integral_constant<int, 3>{});
+		static_for<0, NBATCH>(pv_batch);
 		// issue order: every product of a batch but the last is followed by the two transposed reads
 		// of one fragment of the next batch (left to itself the compiler's order, and with it the
 		// kernel's duration, changes with unrelated edits)
@@ -662,7 +660,6 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 		}
 		__builtin_amdgcn_sched_group_barrier(0x008, NF * QB, 0);
 		__builtin_amdgcn_sched_barrier(0);
-		static_assert(NBATCH <= 4, "");
 	};
 
 	// One pipeline step: publish tile t, start the copies of tile t + 1, compute.
@@ -687,9 +684,9 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 		if (!skip) tile_body(masked_tag, n0);
 		// the other buffers next time
 #pragma unroll
-		for (int ks = 0; ks < KS; ++ks) koff[ks] ^= TILE_BYTES;
+		for (int ks = 0; ks < KR; ++ks) koff[ks] ^= TILE_BYTES;
 #pragma unroll
-		for (int db = 0; db < DB; ++db) {
+		for (int db = 0; db < DR; ++db) {
 			voff[db][0] ^= TILE_BYTES;
 			voff[db][1] ^= TILE_BYTES;
 		}
