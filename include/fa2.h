@@ -135,6 +135,20 @@ typedef struct fa2_params {
 	 * place of scale q.k, before bias and masks, as in the reference's naive attention
 	 * (refrence_call.py:33,48-51); the backward carries the factor 1 - tanh^2.  0 = off.      */
 	float softcap;
+
+	/* Optional gradient of the additive bias (backward only; requires `bias` or `softcap`, i.e. the kernel
+	 * variants that carry an additive term).  fp32 [B, Hq, Sq, Sk] with the element strides given, unit
+	 * stride on Sk, 16-byte aligned with strides that are multiples of 4: receives, per (batch, q-head),
+	 *   dbias[b, h, i, j] = P[i, j] * (dP[i, j] - delta[i]),
+	 * the gradient with respect to the term added to the score (before the softmax scale reaches dQ / dK and
+	 * before the 1 - tanh^2 factor of soft-capping).  A bias that is broadcast over batch or heads has the
+	 * sum of these entries over the broadcast axes as its gradient; that reduction is the caller's (one
+	 * `sum`), so the kernel needs no atomics and stays deterministic.  The dQ kernel writes it, tile by tile:
+	 * positions of key tiles it skips (beyond a length, outside the window or the causal range) are not
+	 * written - pass a zero-filled buffer.  The reference returns no gradient for its bias
+	 * (_flash_attention.py:88), so this has no counterpart there. */
+	float* dbias;
+	int64_t dbias_stride_b, dbias_stride_h, dbias_stride_m;
 } fa2_params;
 
 /* sizeof(fa2_params) in the first version of this header: up to and including scratch_bytes */

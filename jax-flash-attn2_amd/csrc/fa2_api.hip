@@ -85,6 +85,12 @@ int validate(const fa2_params* p, int which, bool own_scratch = false) {
 		if ((rc = check_tensor(p->dq, true))) return rc;
 		if ((rc = check_tensor(p->dk, true))) return rc;
 		if ((rc = check_tensor(p->dv, true))) return rc;
+		if (p->dbias) {
+			if (!p->bias && !(p->softcap > 0.f)) return FA2_EINVAL_BIAS;
+			if (!aligned16(p->dbias)) return FA2_EINVAL_BIAS;
+			if (p->dbias_stride_b < 0 || p->dbias_stride_h < 0 || p->dbias_stride_m < p->Sk) return FA2_EINVAL_BIAS;
+			if (p->dbias_stride_b % 4 || p->dbias_stride_h % 4 || p->dbias_stride_m % 4) return FA2_EINVAL_BIAS;
+		}
 		size_t need = fa2_bwd_scratch_bytes(p);
 		if (own_scratch) {
 			if (need > FA2_STATIC_SCRATCH_BYTES) return FA2_ESCRATCH_STATIC;
@@ -257,6 +263,10 @@ static int bwd_launch(const fa2_params* p, void* hip_stream, int stages, void* s
 	a.dk = conv(p->dk);
 	a.dv = conv(p->dv);
 	a.delta = (float*)scratch_ptr;
+	a.dbias = (char*)p->dbias;
+	a.dbias_sb = p->dbias_stride_b * 4;
+	a.dbias_sh = p->dbias_stride_h * 4;
+	a.dbias_sm = p->dbias_stride_m * 4;
 	hipError_t e = fa2::launch_bwd(p->dtype, p->D, p->bias != nullptr || p->softcap > 0.f, p->p_drop > 0.f, a, (hipStream_t)hip_stream);
 	return e == hipSuccess ? FA2_OK : FA2_EHIP;
 }

@@ -1057,6 +1057,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 #pragma unroll
 				for (int aa = 0; aa < 4; ++aa) {
 					u32x4 rnd;
+					float dcap[4];
 					if constexpr (DROP) {
 						int j4 = (n0 + 32 * kb + 8 * aa + 4 * g) >> 2;
 						rnd = philox4x32_10((uint32_t)j4, (uint32_t)qrow[qb], (uint32_t)h, (uint32_t)b, drop_k0, drop_k1);
@@ -1079,7 +1080,27 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 						float dpe = dp[qb][i];
 						if constexpr (DROP) dpe = rnd[e] >= a.drop_thr ? dpe * a.drop_inv_keep : 0.f;
 						s[qb][i] = FOLD_DP ? p * dpe : p * (dpe - del_r[qb]);
-						if constexpr (CAP) s[qb][i] *= __builtin_fmaf(-th, th, 1.f);  // d tanh
+						if constexpr (CAP) dcap[e] = __builtin_fmaf(-th, th, 1.f);  // d tanh
+					}
+					if constexpr (BIAS) {
+						// gradient of the additive term: this lane's row, keys j0 .. j0 + 3 (wave-uniform branch)
+						if (a.dbias) {
+							int j0 = n0 + 32 * kb + 8 * aa + 4 * g;
+							if (qrow[qb] < a.Sq && j0 < a.Sk) {
+								char* dp_ = a.dbias + (int64_t)b * a.dbias_sb + (int64_t)h * a.dbias_sh + (int64_t)qrow[qb] * a.dbias_sm + (int64_t)j0 * 4;
+								if (j0 + 3 < a.Sk) {
+									*(f32x4*)dp_ = f32x4{s[qb][4 * aa], s[qb][4 * aa + 1], s[qb][4 * aa + 2], s[qb][4 * aa + 3]};
+								} else {
+#pragma unroll
+									for (int e = 0; e < 4; ++e)
+										if (j0 + e < a.Sk) ((float*)dp_)[e] = s[qb][4 * aa + e];
+								}
+							}
+						}
+					}
+					if constexpr (CAP) {
+#pragma unroll
+						for (int e = 0; e < 4; ++e) s[qb][4 * aa + e] *= dcap[e];
 					}
 				}
 #pragma unroll

@@ -23,6 +23,8 @@ struct KArgs {
 	int bias_vec4;   // rows are 4-element aligned: vector loads allowed
 	float mask_fill; // FA2_MASK_U8: the additive value of a masked position = lowest finite value of the element type
 	int bias_lds;    // bias tiles may be copied global->LDS in 16-byte pieces (see fa2_api.hip)
+	char* dbias;     // backward, optional: fp32 [B, Hq, Sq, Sk] gradient of the additive term (dQ kernel variants with bias)
+	int64_t dbias_sb, dbias_sh, dbias_sm;  // bytes
 	const int32_t* seqlens;
 	const int32_t* kv_lens;  // [B]: keys at or beyond kv_lens[b] are masked (query rows unaffected)
 	int B, Sq, Sk, Hq, Hkv;

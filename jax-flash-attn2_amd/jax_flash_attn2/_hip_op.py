@@ -173,8 +173,9 @@ def fwd(q, k, v, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, 
 
 
 def bwd(q, k, v, out, lse, dout, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, causal=False,
-        dropout_seed=None, kv_lens=None, window=None, softcap=0.0):
-	"""Returns (dq, dk, dv) in the dtypes of q, k, v; dk/dv summed over each KV group."""
+        dropout_seed=None, kv_lens=None, window=None, softcap=0.0, need_dbias=False):
+	"""Returns (dq, dk, dv) in the dtypes of q, k, v; dk/dv summed over each KV group.  With `need_dbias` a fourth
+	result: the gradient of the additive bias, fp32, in the shape of `bias` (summed over the axes it is broadcast on)."""
 	lib = _lib.load()
 	D0 = q.shape[-1]
 	D = _kernel_head_dim(D0)
@@ -194,10 +195,36 @@ def bwd(q, k, v, out, lse, dout, bias=None, seqlens=None, softmax_scale=None, dr
 	scratch = torch.empty((max(need, 256),), dtype=torch.uint8, device=q.device)
 	p.scratch = scratch.data_ptr()
 	p.scratch_bytes = scratch.numel()
+	dbias = None
+	if need_dbias:
+		if bias is None or bias.dtype == torch.uint8:
+			raise ValueError("the bias gradient needs a floating-point bias")
+		# the kernel writes the per-(batch, head) gradient and leaves skipped key tiles alone: zero-filled
+		dbias = torch.zeros((B, Hq, Sq, k.shape[1]), dtype=torch.float32, device=q.device)
+		if dbias.shape[3] % 4:  # rows must start on 16 bytes
+			dbias = torch.zeros((B, Hq, Sq, (k.shape[1] + 3) // 4 * 4), dtype=torch.float32, device=q.device)[..., : k.shape[1]]
+		p.dbias = dbias.data_ptr()
+		p.dbias_stride_b, p.dbias_stride_h, p.dbias_stride_m = dbias.stride(0), dbias.stride(1), dbias.stride(2)
 	_lib.check(lib.fa2_bwd(ctypes.byref(p), _stream_ptr(q.device)))
 	if D != D0:
 		dq, dk, dv = dq[..., :D0], dk[..., :D0], dv[..., :D0]
+	if need_dbias:
+		return dq, dk, dv, _reduce_dbias(dbias, bias.shape, k.shape[2])
 	return dq, dk, dv
+
+
+def _reduce_dbias(full: torch.Tensor, bias_shape, Hkv: int) -> torch.Tensor:
+	"""[B, Hq, Sq, Sk] per-head gradient -> the shape of the bias: summed over the q-heads of a KV group for a bias
+	with Hkv heads, over all heads / batch rows for a size-1 axis (the axes the kernels broadcast the bias on)."""
+	B, Hq = full.shape[:2]
+	Bb, Hb = bias_shape[0], bias_shape[1]
+	if Hb == 1:
+		full = full.sum(dim=1, keepdim=True)
+	elif Hb != Hq:
+		full = full.reshape(B, Hkv, Hq // Hkv, *full.shape[2:]).sum(dim=2)
+	if Bb == 1 and B != 1:
+		full = full.sum(dim=0, keepdim=True)
+	return full
 
 
 def dropout_mask(B, H, Sq, Sk, dropout_prob, dropout_seed, device) -> torch.Tensor:
@@ -263,7 +290,9 @@ class Plan:
 class _FlashAttentionFn(torch.autograd.Function):
 	"""Differentiation rule; the torch spelling of the reference's
 	`flash_attention_call.defvjp(_jax_fwd_attention_call, _jax_bwd_attention_call)`
-	(_flash_attention.py:119-122).  Returns (dq, dk, dv) and None for everything else."""
+	(_flash_attention.py:119-122).  Returns (dq, dk, dv) and None for everything else - except the bias: where
+	the reference returns None for it (_flash_attention.py:88), a floating-point bias that requires a gradient
+	gets one here."""
 
 	@staticmethod
 	def forward(ctx, q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens=None, window=None, softcap=0.0):
@@ -276,8 +305,11 @@ class _FlashAttentionFn(torch.autograd.Function):
 	def backward(ctx, dout):
 		q, k, v, bias, seqlens, out, lse, kv_lens = ctx.saved_tensors
 		softmax_scale, dropout_prob, causal, dropout_seed, window, softcap = ctx.cfg
-		dq, dk, dv = bwd(q, k, v, out, lse, dout, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens, window, softcap)
-		return dq, dk, dv, None, None, None, None, None, None, None, None, None
+		need_dbias = bias is not None and ctx.needs_input_grad[3]
+		res = bwd(q, k, v, out, lse, dout, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens, window, softcap,
+		          need_dbias=need_dbias)
+		dbias = res[3].to(bias.dtype) if need_dbias else None
+		return res[0], res[1], res[2], dbias, None, None, None, None, None, None, None, None
 
 
 def flash_attention(

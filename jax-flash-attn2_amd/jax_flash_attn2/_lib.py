@@ -63,6 +63,10 @@ class Fa2Params(ctypes.Structure):
 		("window_left", ctypes.c_int32),
 		("window_right", ctypes.c_int32),
 		("softcap", ctypes.c_float),
+		("dbias", ctypes.c_void_p),
+		("dbias_stride_b", ctypes.c_int64),
+		("dbias_stride_h", ctypes.c_int64),
+		("dbias_stride_m", ctypes.c_int64),
 	]
 
 

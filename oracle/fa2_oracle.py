@@ -233,11 +233,14 @@ def attention_fwd(q, k, v, bias=None, causal=False, scale=None, seqlens=None,
 
 
 def attention_bwd(q, k, v, dO, bias=None, causal=False, scale=None, seqlens=None,
-                  p_drop=0.0, seed=0, dtype=np.float64, pos_offset=(0, 0, 0), kv_lens=None, window=None, softcap=0.0):
+                  p_drop=0.0, seed=0, dtype=np.float64, pos_offset=(0, 0, 0), kv_lens=None, window=None, softcap=0.0,
+                  return_dbias=False):
 	"""Analytic gradients (dQ, dK, dV) of sum(O * dO); FlashAttention-2 Algorithm 2,
 	the same five products as flash_attention_jax/_backward_jax.py:111-127, with
 	dK/dV summed over the q-heads of each KV group (_backward_triton.py:1156-1161).
-	No gradient for bias / mask / seed (_flash_attention.py:88, _backward_jax.py:164)."""
+	No gradient for mask / seed (_flash_attention.py:88, _backward_jax.py:164).  The reference returns none for the
+	bias either; `return_dbias` adds it as a fourth result: dS = P (dP - delta) before the scale, summed over the
+	axes the bias is broadcast on (a size-1 batch or head axis, the q-heads of a KV group for a bias with Hkv heads)."""
 	B, Sq, Hq, D = q.shape
 	Sk, Hkv = k.shape[1], k.shape[2]
 	scale = (1.0 / math.sqrt(D)) if scale is None else scale
@@ -256,6 +259,16 @@ def attention_bwd(q, k, v, dO, bias=None, causal=False, scale=None, seqlens=None
 		dp = dpd
 	delta = np.einsum("bihd,bihd->bhi", o, dOf)[..., None]  # = rowsum(P * dP)
 	ds = p * (dp - delta)
+	dbias = None
+	if return_dbias:
+		dbias = ds  # [B, Hq, Sq, Sk]
+		bshape = np.shape(bias)
+		if bshape[1] == 1:
+			dbias = dbias.sum(axis=1, keepdims=True)
+		elif bshape[1] != Hq:
+			dbias = dbias.reshape(B, Hkv, r, Sq, Sk).sum(axis=2)
+		if bshape[0] == 1 and B != 1:
+			dbias = dbias.sum(axis=0, keepdims=True)
 	if softcap and softcap > 0:
 		# d/dx [c tanh(x / c)] = 1 - tanh^2(x / c)
 		th = _scores(q, k, None, scale, False, None, dtype, softcap=softcap, return_tanh=True)[3]
@@ -264,6 +277,8 @@ def attention_bwd(q, k, v, dO, bias=None, causal=False, scale=None, seqlens=None
 	dk_full = _ptx(ds, qf) * dtype(scale)
 	dk = dk_full.reshape(B, Sk, Hkv, r, D).sum(axis=3)
 	dv = dv_full.reshape(B, Sk, Hkv, r, D).sum(axis=3)
+	if return_dbias:
+		return dq, dk, dv, dbias
 	return dq, dk, dv
 
 

@@ -38,9 +38,10 @@ def test_struct_layout_matches_c():
 #include <stddef.h>
 #include "fa2.h"
 int main(void) {
-  printf("%zu %zu %zu %zu %zu %zu %zu %zu %zu\n", sizeof(fa2_params), offsetof(fa2_params, seed), offsetof(fa2_params, q),
+  printf("%zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu\n", sizeof(fa2_params), offsetof(fa2_params, seed), offsetof(fa2_params, q),
          offsetof(fa2_params, lse), offsetof(fa2_params, bias), offsetof(fa2_params, bias_stride_b),
-         offsetof(fa2_params, seqlens), offsetof(fa2_params, dout), offsetof(fa2_params, scratch));
+         offsetof(fa2_params, seqlens), offsetof(fa2_params, dout), offsetof(fa2_params, scratch),
+         offsetof(fa2_params, softcap), offsetof(fa2_params, dbias), offsetof(fa2_params, dbias_stride_m));
   return 0;
 }"""
 	with tempfile.TemporaryDirectory() as d:
@@ -50,7 +51,7 @@ int main(void) {
 		subprocess.check_call(["gcc", "-I", os.path.join(ROOT, "include"), c, "-o", exe])
 		got = [int(x) for x in subprocess.check_output([exe]).split()]
 	P = _lib.Fa2Params
-	want = [ctypes.sizeof(P)] + [getattr(P, f).offset for f in ("seed", "q", "lse", "bias", "bias_stride_b", "seqlens", "dout", "scratch")]
+	want = [ctypes.sizeof(P)] + [getattr(P, f).offset for f in ("seed", "q", "lse", "bias", "bias_stride_b", "seqlens", "dout", "scratch", "softcap", "dbias", "dbias_stride_m")]
 	assert got == want
 
 
@@ -141,6 +142,26 @@ def test_validate_backward_scratch():
 	assert lib.fa2_bwd(ctypes.byref(p), None) == -5
 	assert lib.fa2_fwd(None, None) == -1
 	assert lib.fa2_dropout_mask(ctypes.byref(p), None, None) == -5
+
+
+def test_validate_bias_gradient_buffer():
+	def with_dbias(**kw):
+		p = _good_params()
+		p.bias, p.bias_dtype, p.bias_stride_m = 0x40000, 2, 128
+		p.dbias = 0x50000
+		p.dbias_stride_b, p.dbias_stride_h, p.dbias_stride_m = 8 * 128 * 128, 128 * 128, 128
+		for k, v in kw.items():
+			setattr(p, k, v)
+		return p
+
+	assert _rc(with_dbias(), 1) == 0
+	assert _rc(with_dbias(), 0) == 0                       # the forward does not look at it
+	assert _rc(with_dbias(bias=0), 1) == -8                # no additive term in the kernels: nothing to differentiate
+	assert _rc(with_dbias(bias=0, softcap=2.0), 1) == 0    # ... unless soft-capping selects the variants that carry one
+	assert _rc(with_dbias(dbias=0x50004), 1) == -8         # rows are stored 16 bytes at a time
+	assert _rc(with_dbias(dbias_stride_m=126), 1) == -8
+	assert _rc(with_dbias(dbias_stride_m=64), 1) == -8     # shorter than a row
+	assert _rc(with_dbias(dbias_stride_h=-4), 1) == -8
 
 
 def test_missing_library_fails_loudly(monkeypatch):

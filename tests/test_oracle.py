@@ -161,6 +161,33 @@ def test_backward_matches_finite_differences(kw):
 		assert np.abs(num - g).max() < 1e-7
 
 
+@pytest.mark.parametrize("bshape", [(2, 4), (2, 2), (2, 1), (1, 4), (1, 1)], ids=["bBhH", "bBhKV", "bBh1", "b1hH", "b1h1"])
+@pytest.mark.parametrize("kw", [dict(), dict(causal=True, p_drop=0.3, seed=7), dict(softcap=0.8, window=(3, 1))])
+def test_bias_gradient_matches_finite_differences(bshape, kw):
+	"""dbias of attention_bwd(return_dbias=True) against central differences in the entries of the bias, for every
+	broadcast shape of the bias (the gradient of a broadcast entry is the sum over the positions it feeds)."""
+	rng = np.random.default_rng(11)
+	B, Sq, Sk, Hq, Hkv, D = 2, 5, 6, 4, 2, 4
+	q, k, v, dO = _rand(rng, B, Sq, Sk, Hq, Hkv, D)
+	bias = rng.normal(size=(*bshape, Sq, Sk))
+	dbias = O.attention_bwd(q, k, v, dO, bias=bias, return_dbias=True, **kw)[3]
+	assert dbias.shape == bias.shape
+	f = lambda bb: np.sum(O.attention_fwd(q, k, v, bias=bb, **kw)[0] * dO)
+	eps = 1e-6
+	num = np.zeros_like(bias)
+	it = np.nditer(bias, flags=["multi_index"])
+	for _ in it:
+		mi = it.multi_index
+		a, b = bias.copy(), bias.copy()
+		a[mi] += eps
+		b[mi] -= eps
+		num[mi] = (f(a) - f(b)) / (2 * eps)
+	assert np.abs(num - dbias).max() < 1e-7
+	# the first three results do not depend on the flag
+	for x, y in zip(O.attention_bwd(q, k, v, dO, bias=bias, **kw), O.attention_bwd(q, k, v, dO, bias=bias, return_dbias=True, **kw)):
+		assert np.array_equal(x, y)
+
+
 def test_backward_identities():
 	rng = np.random.default_rng(6)
 	q, k, v, dO = _rand(rng, 1, 12, 12, 4, 2, 8)

@@ -404,6 +404,53 @@ def test_mask_as_finfo_min_bias():
 	assert g[1][0, 100:].abs().max().item() == 0 and g[2][0, 100:].abs().max().item() == 0
 
 
+@pytest.mark.parametrize(
+	"bshape", [(1, 1), (2, 1), (1, 4), (2, 4), (2, 2)], ids=["b1h1", "bBh1", "b1hH", "bBhH", "bBhKV"]
+)
+@pytest.mark.parametrize("D,dtype", [(64, torch.bfloat16), (128, torch.float16), (256, torch.bfloat16)])
+def test_bias_gradient(bshape, D, dtype):
+	"""fa2_params.dbias (the dQ kernel writes the per-head gradient of the additive term, the operator sums it over the
+	axes the bias is broadcast on) against the oracle; ragged tiles, causal, dropout, key lengths; dq / dk / dv unchanged."""
+	B, Sq, Sk, Hq, Hkv = 2, 160, 203, 4, 2
+	for causal, p, kv_lens in ((False, 0.0, None), (True, 0.2, None), (False, 0.0, [150, 64])):
+		q, k, v, do, bias = make_inputs(B, Sq, Sk, Hq, Hkv, D, dtype, 5, (*bshape, Sq, Sk))
+		kw = dict(causal=causal, p_drop=p, seed=9, kv_lens=kv_lens)
+		ref = O.attention_bwd(f64(q), f64(k), f64(v), f64(do), f64(bias), return_dbias=True, **kw)
+		kl = None if kv_lens is None else torch.tensor(kv_lens, dtype=torch.int32, device=DEV)
+		o, lse = op.fwd(_dev(q), _dev(k), _dev(v), _dev(bias), None, None, p, causal, 9, kv_lens=kl)
+		g = op.bwd(_dev(q), _dev(k), _dev(v), o, lse, _dev(do), _dev(bias), None, None, p, causal, 9, kv_lens=kl, need_dbias=True)
+		g0 = op.bwd(_dev(q), _dev(k), _dev(v), o, lse, _dev(do), _dev(bias), None, None, p, causal, 9, kv_lens=kl)
+		torch.cuda.synchronize()
+		what = f"bias {bshape} D{D} causal={causal} p={p} kv_lens={kv_lens}"
+		check_grads(g[:3], ref[:3], what)
+		for a, b in zip(g[:3], g0):
+			assert torch.equal(a, b), what
+		db = g[3].cpu().numpy()
+		assert db.shape == ref[3].shape and np.isfinite(db).all(), what
+		e = O.rel_l2(db, ref[3])
+		assert e <= 1e-2, f"{what}: dbias rel-L2 {e:.3e}"
+
+
+def test_bias_gradient_through_autograd_and_softcap():
+	"""A bias that requires a gradient gets one from the operator's differentiation rule (the reference returns None for
+	it, _flash_attention.py:88); with soft-capping the bias gradient does not carry the 1 - tanh^2 factor."""
+	B, Sq, Sk, Hq, Hkv, D = 1, 96, 130, 4, 4, 64
+	q, k, v, do, bias = make_inputs(B, Sq, Sk, Hq, Hkv, D, torch.bfloat16, 2, (1, 1, Sq, Sk), bias_dtype=torch.float32)
+	ref = O.attention_bwd(f64(q), f64(k), f64(v), f64(do), f64(bias), causal=True, softcap=2.0, return_dbias=True)
+	qd, kd, vd, bd = (_dev(t).requires_grad_(True) for t in (q, k, v, bias))
+	out = op.flash_attention(qd, kd, vd, bias=bd, causal=True, softcap=2.0)
+	out.backward(_dev(do))
+	torch.cuda.synchronize()
+	check_grads((qd.grad, kd.grad, vd.grad), ref[:3], "autograd with bias gradient")
+	assert bd.grad.shape == bias.shape and bd.grad.dtype == torch.float32
+	assert O.rel_l2(bd.grad.cpu().numpy(), ref[3]) <= 1e-2
+	# no gradient asked for the bias: none computed
+	qd2 = _dev(q).requires_grad_(True)
+	b2 = _dev(bias)
+	op.flash_attention(qd2, _dev(k), _dev(v), bias=b2, causal=True, softcap=2.0).backward(_dev(do))
+	assert b2.grad is None and torch.equal(qd2.grad, qd.grad)
+
+
 @pytest.mark.parametrize("causal", [False, True])
 def test_seqlens(causal):
 	_run_case(4, 256, 256, 4, 2, 128, torch.bfloat16, causal=causal, seqlens=[256, 100, 1, 0])
