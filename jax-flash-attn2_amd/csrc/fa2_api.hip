@@ -101,9 +101,10 @@ int validate(const fa2_params* p, int which, bool own_scratch = false) {
 	return FA2_OK;
 }
 
+// an element is kept iff its 16-bit value is >= this
 uint32_t drop_threshold(float p) {
-	double t = floor((double)p * 4294967296.0);
-	return t >= 4294967295.0 ? 0xFFFFFFFFu : (uint32_t)t;
+	double t = floor((double)p * 65536.0);
+	return t >= 65535.0 ? 0xFFFFu : (uint32_t)t;
 }
 
 void fill(const fa2_params* p, KArgs& a) {

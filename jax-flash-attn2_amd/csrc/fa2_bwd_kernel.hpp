@@ -175,6 +175,16 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		}
 	}
 
+	// The fragments must have arrived before the loop over streamed tiles starts.  Otherwise the compiler places its
+	// waits for these loads (s_waitcnt vmcnt) at their first uses inside the loop - it does not see the wait that
+	// publishes a tile - where the same counter also counts the tile copies in flight: every step would then wait
+	// for the copies of the NEXT tile before its first product.  (With KV_AGPR the moves into the accumulation
+	// registers below are that point.)
+	if constexpr (!KV_AGPR) {
+#pragma unroll
+		for (int ks = 0; ks < KS; ++ks) asm volatile("; K / V fragment present" : "+v"(kf[ks]), "+v"(vf[ks]));
+	}
+
 	f32x16 dk[DB], dv[DB];
 #pragma unroll
 	for (int db = 0; db < DB; ++db)
@@ -439,21 +449,23 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		// the previous one's full pipeline latency).
 		float bx[4][4], by[4][4];
 		float bt[4][4];  // CAP: tanh of the scaled score, for the factor 1 - tanh^2 of its derivative
-		// dropout keep bits of a quad (bit e = value 4q + e), produced one value per slot while
-		// the previous quad is processed: one Philox call at a time keeps its registers few
+		// dropout keep bits of a quad (bit e = value 4q + e), produced while the previous quad is processed.
+		// One generator call yields the values of 2 adjacent rows x 4 adjacent keys, and the 4 lanes of a
+		// DPP quad hold 4 adjacent keys: one call per lane covers the 2 x 4 rows of the quads q and q + 1 (q even) -
+		// lane t evaluates the rows 2 (t & 1), 2 (t & 1) + 1 of quad q + t / 2, reduces its 8 values to 8 keep bits
+		// (bit = value index = 4 (row & 1) + (key & 3)), and the quad exchanges them (DPP broadcasts).  The call is
+		// cut into 4 parts (rounds 0-2, 3-5, 6-7, 8-9 + exchange) that run in the four micro-step slots of the
+		// quad before q; the odd quads' slots stay free of generator work.
 		uint32_t keepw[4] = {0u, 0u, 0u, 0u};
-		// One generator call yields the words of 4 adjacent keys of one row, and the 4 lanes of a
-		// quad hold 4 adjacent keys: lane t of a quad evaluates row e = t of the quad of rows,
-		// reduces its 4 words to 4 keep bits, and the quad exchanges them (DPP broadcasts).  The
-		// call is cut into 4 parts (rounds 0-2, 3-5, 6-7, 8-9 + exchange) that run in the four
-		// micro-step slots of the previous quad.  `u` selects one of two calls in flight.
 		uint32_t phs[2][4];
 		auto keep_bit = [&](int qb, int q, int part, int u = 0) __attribute__((always_inline)) {
 			if constexpr (DROP) {
+				if (q & 1) return;
 				uint32_t(&cs)[4] = phs[u];
 				if (part == 0) {
+					const int t = c & 3;
 					cs[0] = (uint32_t)(jcol >> 2);
-					cs[1] = (uint32_t)(m0 + 32 * qb + 8 * q + 4 * g + (c & 3));
+					cs[1] = (uint32_t)((m0 + 32 * qb + 8 * (q + (t >> 1)) + 4 * g + 2 * (t & 1)) >> 1);
 					cs[2] = (uint32_t)hq;
 					cs[3] = (uint32_t)b;
 					philox4x32_rounds<0, 3>(cs, drop_k0, drop_k1);
@@ -463,16 +475,17 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 					philox4x32_rounds<6, 8>(cs, drop_k0, drop_k1);
 				} else {
 					philox4x32_rounds<8, 10>(cs, drop_k0, drop_k1);
-					// bit t = key (jcol & ~3) + t of this lane's row is kept
-					uint32_t mine = (cs[0] >= a.drop_thr ? 1u : 0u) | (cs[1] >= a.drop_thr ? 2u : 0u) | (cs[2] >= a.drop_thr ? 4u : 0u) |
-					                (cs[3] >= a.drop_thr ? 8u : 0u);
-					// row e was evaluated by lane e of the quad; this lane's key is bit c & 3 of its mask
+					uint32_t mine = 0;
+#pragma unroll
+					for (int v = 0; v < 8; ++v) mine |= keep16(cs[v >> 1], v & 1, a.drop_thr) ? (1u << v) : 0u;
+					// rows e = 0, 1 of quad q were evaluated by lane 0 of the quad, e = 2, 3 by lane 1; quad q + 1: lanes 2, 3
 					uint32_t r0 = (uint32_t)__builtin_amdgcn_mov_dpp((int)mine, 0x00, 0xf, 0xf, false);
 					uint32_t r1 = (uint32_t)__builtin_amdgcn_mov_dpp((int)mine, 0x55, 0xf, 0xf, false);
 					uint32_t r2 = (uint32_t)__builtin_amdgcn_mov_dpp((int)mine, 0xaa, 0xf, 0xf, false);
 					uint32_t r3 = (uint32_t)__builtin_amdgcn_mov_dpp((int)mine, 0xff, 0xf, 0xf, false);
-					const uint32_t sh = (uint32_t)(c & 3);
-					keepw[q & 3] = ((r0 >> sh) & 1u) | (((r1 >> sh) & 1u) << 1) | (((r2 >> sh) & 1u) << 2) | (((r3 >> sh) & 1u) << 3);
+					const uint32_t sh = (uint32_t)(c & 3);  // this lane's key among the call's four
+					keepw[q & 3] = ((r0 >> sh) & 1u) | (((r0 >> (4 + sh)) & 1u) << 1) | (((r1 >> sh) & 1u) << 2) | (((r1 >> (4 + sh)) & 1u) << 3);
+					keepw[(q + 1) & 3] = ((r2 >> sh) & 1u) | (((r2 >> (4 + sh)) & 1u) << 1) | (((r3 >> sh) & 1u) << 2) | (((r3 >> (4 + sh)) & 1u) << 3);
 				}
 			}
 		};
@@ -720,6 +733,11 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 			boffq[1] ^= BIAS_BYTES;
 		}
 		if (has_next) store_stat(next_stat, buf ^ 1);
+		// The load of the statistics has completed on every path out of the step.  Without this use the compiler
+		// takes the load for possibly still in flight at the top of the next step (it cannot tell that the two
+		// `has_next` tests agree) and guards the first reuse of its register there with s_waitcnt vmcnt(0) - which
+		// on the hardware waits for the tile copies that were just started.
+		asm volatile("; statistics of the next tile present" ::"v"(next_stat));
 	};
 	// Per q-head the streamed tiles are: tiles crossing this wave's causal diagonal / the window's
 	// right edge (masked), tiles entirely inside (no mask), and tiles on the window's left edge or a
@@ -776,9 +794,11 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 // dQ
 // ---------------------------------------------------------------------------
 // BLDS: the bias goes through LDS as in the forward kernel (conditions checked by the launcher)
-template <typename T, int D, int NW, int QB, int WPS, bool BIAS, bool DROP, bool BLDS = false, bool CAP = false>
+// DBIAS: also writes the gradient of the additive term (a.dbias); on the plain path with bias
+template <typename T, int D, int NW, int QB, int WPS, bool BIAS, bool DROP, bool BLDS = false, bool CAP = false, bool DBIAS = false>
 __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 	static_assert(!CAP || (BIAS && !BLDS), "soft-capping runs on the plain path with bias");
+	static_assert(!DBIAS || (BIAS && !BLDS), "the bias gradient is written on the plain path with bias");
 	typedef typename T::V8 V8;
 	constexpr int BM = NW * QB * 32;
 	constexpr int BN = kFwdBN;
@@ -1054,14 +1074,11 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 			V8 dsf[QB][2];
 #pragma unroll
 			for (int qb = 0; qb < QB; ++qb) {
+				uint32_t dw[4][2];
+				if constexpr (DROP) dropout_words_rowlane<true>(n0 + 32 * kb + 4 * g, (uint32_t)qrow[qb], (uint32_t)h, (uint32_t)b, drop_k0, drop_k1, dw);
 #pragma unroll
 				for (int aa = 0; aa < 4; ++aa) {
-					u32x4 rnd;
 					float dcap[4];
-					if constexpr (DROP) {
-						int j4 = (n0 + 32 * kb + 8 * aa + 4 * g) >> 2;
-						rnd = philox4x32_10((uint32_t)j4, (uint32_t)qrow[qb], (uint32_t)h, (uint32_t)b, drop_k0, drop_k1);
-					}
 #pragma unroll
 					for (int e = 0; e < 4; ++e) {
 						int i = 4 * aa + e;
@@ -1078,13 +1095,13 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 							p = ((j <= jmax[qb]) & (j >= jmin[qb])) ? p : 0.f;
 						}
 						float dpe = dp[qb][i];
-						if constexpr (DROP) dpe = rnd[e] >= a.drop_thr ? dpe * a.drop_inv_keep : 0.f;
+						if constexpr (DROP) dpe = keep16(dw[aa][e >> 1], e & 1, a.drop_thr) ? dpe * a.drop_inv_keep : 0.f;
 						s[qb][i] = FOLD_DP ? p * dpe : p * (dpe - del_r[qb]);
 						if constexpr (CAP) dcap[e] = __builtin_fmaf(-th, th, 1.f);  // d tanh
 					}
-					if constexpr (BIAS) {
-						// gradient of the additive term: this lane's row, keys j0 .. j0 + 3 (wave-uniform branch)
-						if (a.dbias) {
+					if constexpr (DBIAS) {
+						// gradient of the additive term: this lane's row, keys j0 .. j0 + 3
+						{
 							int j0 = n0 + 32 * kb + 8 * aa + 4 * g;
 							if (qrow[qb] < a.Sq && j0 < a.Sk) {
 								char* dp_ = a.dbias + (int64_t)b * a.dbias_sb + (int64_t)h * a.dbias_sh + (int64_t)qrow[qb] * a.dbias_sm + (int64_t)j0 * 4;
@@ -1217,7 +1234,11 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 		a.mtiles = (a.Sq + C::DQ_BM - 1) / C::DQ_BM;
 		a.interleave = a.xcd_remap == 1 ? launch_order(a, a.Hq / a.Hkv, groups / 8) : 1;
 		dim3 grid((unsigned)(a.mtiles * a.B * a.Hq)), block(C::DQ_NW * 64);
-		if (BIAS && a.softcap > 0.f)
+		if (BIAS && a.dbias && a.softcap > 0.f)
+			hipLaunchKernelGGL((bwd_dq_kernel<T, D, C::DQ_NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, false, BIAS, BIAS>), grid, block, 0, s, a);
+		else if (BIAS && a.dbias)
+			hipLaunchKernelGGL((bwd_dq_kernel<T, D, C::DQ_NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, false, false, BIAS>), grid, block, 0, s, a);
+		else if (BIAS && a.softcap > 0.f)
 			hipLaunchKernelGGL((bwd_dq_kernel<T, D, C::DQ_NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, false, BIAS>), grid, block, 0, s, a);
 		else if (BIAS && a.bias_lds && D <= 128)
 			hipLaunchKernelGGL((bwd_dq_kernel<T, D, C::DQ_NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, BIAS>), grid, block, 0, s, a);

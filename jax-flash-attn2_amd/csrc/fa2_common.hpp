@@ -317,8 +317,12 @@ struct TileLoader {
 FA2_DEV void wait_async_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // ---------------------------------------------------------------------------
-// Philox-4x32-10.  counter = (j >> 2, i, h, b), key = (seed lo, seed hi);
-// element (i, j) uses word j & 3 and is kept iff word >= threshold.
+// Dropout: Philox-4x32-10, key = (seed lo, seed hi).  One call serves two adjacent rows x four adjacent
+// keys: counter = (j >> 2, i >> 1, h, b); its four words are eight 16-bit values (word w = values 2w in
+// the low half, 2w + 1 in the high half), value (i & 1) * 4 + (j & 3) belongs to element (i, j), which is
+// kept iff value >= floor(p * 65536).  The generator dominates the cost of dropout (20 64-bit multiplies
+// per call), and both register layouts of the scores let the lanes that share a call exchange its words
+// with DPP moves inside a quad, so every lane evaluates half the calls it has values for.
 // ---------------------------------------------------------------------------
 FA2_DEV u32x4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1) {
 #pragma unroll
@@ -357,6 +361,42 @@ FA2_DEV void philox4x32_rounds(uint32_t (&c)[4], uint32_t k0, uint32_t k1) {
 		c[1] = lo1;
 		c[2] = n2;
 		c[3] = lo0;
+	}
+}
+
+// value `half` (0 / 1) of a word against the threshold
+FA2_DEV bool keep16(uint32_t word, int half, uint32_t thr16) { return (half ? (word >> 16) : (word & 0xffffu)) >= thr16; }
+
+// the neighbouring lane's value (lanes 0 <-> 1, 2 <-> 3 of every quad)
+FA2_DEV uint32_t quad_swap1(uint32_t x) { return (uint32_t)__builtin_amdgcn_mov_dpp((int)x, 0xB1, 0xf, 0xf, false); }
+
+// Layout "lane = query row" (forward and dQ kernels: a lane holds keys jb + 8 aa + e, aa = 0..3, e = 0..3, of its row,
+// and the lane next to it holds the same keys of the other row of the pair): w[aa][0..1] receive the two words with
+// the row's four values for keys jb + 8 aa .. + 3.  SHARE: the lane of the even row evaluates the calls of aa = 0, 2,
+// the lane of the odd row those of aa = 1, 3, and they exchange (needs lane ^ 1 = row ^ 1 in the same (b, h));
+// otherwise every lane evaluates its four calls itself.
+template <bool SHARE>
+FA2_DEV void dropout_words_rowlane(int jb, uint32_t row, uint32_t h, uint32_t b, uint32_t k0, uint32_t k1, uint32_t (&w)[4][2]) {
+	const bool odd = row & 1u;
+	if constexpr (SHARE) {
+#pragma unroll
+		for (int pr = 0; pr < 2; ++pr) {
+			int aa_mine = 2 * pr + (odd ? 1 : 0);
+			u32x4 r = philox4x32_10((uint32_t)((jb + 8 * aa_mine) >> 2), row >> 1, h, b, k0, k1);
+			uint32_t own0 = odd ? r[2] : r[0], own1 = odd ? r[3] : r[1];
+			uint32_t got0 = quad_swap1(odd ? r[0] : r[2]), got1 = quad_swap1(odd ? r[1] : r[3]);
+			w[2 * pr][0] = odd ? got0 : own0;
+			w[2 * pr][1] = odd ? got1 : own1;
+			w[2 * pr + 1][0] = odd ? own0 : got0;
+			w[2 * pr + 1][1] = odd ? own1 : got1;
+		}
+	} else {
+#pragma unroll
+		for (int aa = 0; aa < 4; ++aa) {
+			u32x4 r = philox4x32_10((uint32_t)((jb + 8 * aa) >> 2), row >> 1, h, b, k0, k1);
+			w[aa][0] = odd ? r[2] : r[0];
+			w[aa][1] = odd ? r[3] : r[1];
+		}
 	}
 }
 

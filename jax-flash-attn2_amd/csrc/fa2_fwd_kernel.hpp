@@ -477,15 +477,16 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 		auto pack_p = [&](int qb) __attribute__((always_inline)) {
 			if constexpr (DROP) {
 #pragma unroll
-				for (int kb = 0; kb < KB; ++kb)
+				for (int kb = 0; kb < KB; ++kb) {
+					uint32_t dw[4][2];
+					// (split forward: the rows of a tile may belong to several heads - no sharing between lanes)
+					dropout_words_rowlane<!SPLIT>(n0 + 32 * kb + 4 * g, (uint32_t)qrow[qb], (uint32_t)hl[qb], (uint32_t)b, drop_k0, drop_k1, dw);
 #pragma unroll
-					for (int aa = 0; aa < 4; ++aa) {
-						int j4 = (n0 + 32 * kb + 8 * aa + 4 * g) >> 2;
-						u32x4 rnd = philox4x32_10((uint32_t)j4, (uint32_t)qrow[qb], (uint32_t)hl[qb], (uint32_t)b, drop_k0, drop_k1);
+					for (int aa = 0; aa < 4; ++aa)
 #pragma unroll
 						for (int e = 0; e < 4; ++e)
-							s[kb][qb][4 * aa + e] = rnd[e] >= a.drop_thr ? s[kb][qb][4 * aa + e] : 0.f;
-					}
+							s[kb][qb][4 * aa + e] = keep16(dw[aa][e >> 1], e & 1, a.drop_thr) ? s[kb][qb][4 * aa + e] : 0.f;
+				}
 			}
 #pragma unroll
 			for (int kb = 0; kb < KB; ++kb)

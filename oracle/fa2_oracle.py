@@ -70,18 +70,20 @@ def philox4x32_10(c0, c1, c2, c3, k0, k1):
 
 
 def dropout_threshold(p_drop: float) -> int:
-	"""Integer threshold: an element is kept iff its 32-bit Philox word >= threshold."""
+	"""Integer threshold: an element is kept iff its 16-bit Philox value >= threshold."""
 	if not (0.0 <= p_drop < 1.0):
 		raise ValueError(f"invalid dropout {p_drop}")
-	return min(int(math.floor(float(np.float32(p_drop)) * 4294967296.0)), 0xFFFFFFFF)
+	return min(int(math.floor(float(np.float32(p_drop)) * 65536.0)), 0xFFFF)
 
 
 def dropout_keep_mask(seed: int, p_drop: float, B: int, H: int, Sq: int, Sk: int, pos_offset=(0, 0, 0)) -> np.ndarray:
 	"""keep[b,h,i,j] (bool).  `pos_offset` = (b0, h0, i0) shifts the batch / head /
-	row indices, for checking a slice of a larger problem.
+	row indices, for checking a slice of a larger problem (i0 must be even).
 
-	Counter = (j >> 2, i, h, b), key = (seed & 0xffffffff, seed >> 32); element
-	(i, j) uses output word j & 3 and is kept iff word >= floor(p * 2**32).
+	One generator call serves two adjacent rows x four adjacent keys: counter = (j >> 2, i >> 1, h, b),
+	key = (seed & 0xffffffff, seed >> 32).  Its four 32-bit words are eight 16-bit values (word w holds
+	value 2w in its low half and value 2w + 1 in its high half); element (i, j) owns value
+	(i & 1) * 4 + (j & 3) and is kept iff value >= floor(p * 65536).
 	Position-only: independent of tiling, so forward and both backward kernels
 	regenerate the same mask.  Plays the role of the reference's
 	`tl.rand(seed, offs) > p` (_forward_triton.py:140-143, 325-331).
@@ -89,15 +91,20 @@ def dropout_keep_mask(seed: int, p_drop: float, B: int, H: int, Sq: int, Sk: int
 	thr = np.uint32(dropout_threshold(p_drop))
 	k0 = seed & 0xFFFFFFFF
 	k1 = (seed >> 32) & 0xFFFFFFFF
-	nj4 = (Sk + 3) // 4
-	j4 = np.arange(nj4, dtype=np.uint32)[None, None, None, :]
 	b0, h0, i0 = pos_offset
-	i = (np.arange(Sq, dtype=np.uint32) + np.uint32(i0))[None, None, :, None]
+	if i0 & 1:
+		raise ValueError("row offset must be even (a call serves rows 2m and 2m + 1)")
+	nj4 = (Sk + 3) // 4
+	ni2 = (Sq + 1) // 2
+	j4 = np.arange(nj4, dtype=np.uint32)[None, None, None, :]
+	i2 = (np.arange(ni2, dtype=np.uint32) + np.uint32(i0 // 2))[None, None, :, None]
 	h = (np.arange(H, dtype=np.uint32) + np.uint32(h0))[None, :, None, None]
 	b = (np.arange(B, dtype=np.uint32) + np.uint32(b0))[:, None, None, None]
-	w = philox4x32_10(j4, i, h, b, k0, k1)
-	words = np.stack(w, axis=-1).reshape(B, H, Sq, nj4 * 4)[..., :Sk]
-	return words >= thr
+	w = np.stack(philox4x32_10(j4, i2, h, b, k0, k1), axis=-1)  # [B, H, ni2, nj4, 4]
+	vals = np.stack([w & np.uint32(0xFFFF), w >> np.uint32(16)], axis=-1).reshape(B, H, ni2, nj4, 8)  # value index 2w + half
+	vals = vals.reshape(B, H, ni2, nj4, 2, 4)  # [.., row parity, key & 3]
+	vals = vals.transpose(0, 1, 2, 4, 3, 5).reshape(B, H, ni2 * 2, nj4 * 4)[:, :, :Sq, :Sk]
+	return vals >= thr
 
 
 # --------------------------------------------------------------------------

@@ -34,11 +34,18 @@ def test_dropout_mask_definition_and_rate():
 	B, H, Sq, Sk, p, seed = 2, 3, 37, 50, 0.25, (7 << 32) | 12345
 	keep = O.dropout_keep_mask(seed, p, B, H, Sq, Sk)
 	thr = O.dropout_threshold(p)
-	assert thr == 1 << 30
-	# spot-check single elements against a scalar evaluation of the definition
-	for (b, h, i, j) in [(0, 0, 0, 0), (1, 2, 36, 49), (0, 1, 5, 6), (1, 0, 20, 3)]:
-		w = O.philox4x32_10(np.uint32(j >> 2), np.uint32(i), np.uint32(h), np.uint32(b), seed & 0xFFFFFFFF, seed >> 32)
-		assert bool(keep[b, h, i, j]) == (int(w[j & 3]) >= thr)
+	assert thr == 1 << 14
+	# every element against a scalar evaluation of the definition: one call per (two rows, four keys), eight 16-bit
+	# values, element (i, j) owns value (i & 1) * 4 + (j & 3) = half (v & 1) of word v >> 1
+	for (b, h, i, j) in [(0, 0, 0, 0), (1, 2, 36, 49), (0, 1, 5, 6), (1, 0, 20, 3), (0, 2, 21, 3), (1, 1, 1, 47), (0, 0, 36, 0)]:
+		w = O.philox4x32_10(np.uint32(j >> 2), np.uint32(i >> 1), np.uint32(h), np.uint32(b), seed & 0xFFFFFFFF, seed >> 32)
+		v = (i & 1) * 4 + (j & 3)
+		val = (int(w[v >> 1]) >> 16) if (v & 1) else (int(w[v >> 1]) & 0xFFFF)
+		assert bool(keep[b, h, i, j]) == (val >= thr)
+	# the eight values of one call are used once each: rows (2m, 2m + 1) x keys (4n .. 4n + 3)
+	w = [int(x) for x in O.philox4x32_10(np.uint32(3), np.uint32(4), np.uint32(1), np.uint32(0), seed & 0xFFFFFFFF, seed >> 32)]
+	vals = [(w[v >> 1] >> 16) if (v & 1) else (w[v >> 1] & 0xFFFF) for v in range(8)]
+	assert np.array_equal(keep[0, 1, 8:10, 12:16], (np.array(vals).reshape(2, 4) >= thr))
 	big = O.dropout_keep_mask(42, 0.1, 1, 2, 512, 512)
 	n = big.size
 	assert abs(big.mean() - 0.9) < 4 * np.sqrt(0.09 / n)
