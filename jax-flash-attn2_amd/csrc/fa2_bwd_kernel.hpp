@@ -178,11 +178,14 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	// The fragments must have arrived before the loop over streamed tiles starts.  Otherwise the compiler places its
 	// waits for these loads (s_waitcnt vmcnt) at their first uses inside the loop - it does not see the wait that
 	// publishes a tile - where the same counter also counts the tile copies in flight: every step would then wait
-	// for the copies of the NEXT tile before its first product.  (With KV_AGPR the moves into the accumulation
-	// registers below are that point.)
-	if constexpr (!KV_AGPR) {
+	// for the copies of the NEXT tile before its first product.  (With KV_AGPR the loads go straight into
+	// accumulation registers, where the inline-assembly products read them.)
 #pragma unroll
-		for (int ks = 0; ks < KS; ++ks) asm volatile("; K / V fragment present" : "+v"(kf[ks]), "+v"(vf[ks]));
+	for (int ks = 0; ks < KS; ++ks) {
+		if constexpr (KV_AGPR)
+			asm volatile("; K / V fragment present" : "+a"(kf[ks]), "+a"(vf[ks]));
+		else
+			asm volatile("; K / V fragment present" : "+v"(kf[ks]), "+v"(vf[ks]));
 	}
 
 	f32x16 dk[DB], dv[DB];
