@@ -186,6 +186,8 @@ def main():
 	ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
 	ap.add_argument("--no-cpu-baseline", action="store_true")
 	ap.add_argument("--no-mfma-peak", action="store_true", help="skip the matrix-product-only microbenchmark")
+	ap.add_argument("--no-power-check", action="store_true",
+	                help="skip the rerun of the same launches on all-zero operands (tells whether the timed run was clock-throttled)")
 	ap.add_argument("--copy-calibration", action="store_true",
 	                help="also run a plain 1 GiB device copy (known traffic) so that rocprofv3 FETCH_SIZE / WRITE_SIZE "
 	                     "readings of the attention kernels can be scaled")
@@ -290,6 +292,24 @@ def main():
 		"pct_of_mfma_peak": 100.0 * tflops / peak,
 		"roofline": roofline,
 	}
+	if not args.no_power_check:
+		# The same launches on all-zero q, k, v, dO: the instruction stream, the masks and the memory traffic are those
+		# of the timed run, only the switching activity of the data is gone.  Where this runs faster, the timed run was
+		# held below the 2.4 GHz clock by the chip's power limit, not by the kernels' instruction issue.
+		for t in (q, k, v, do):
+			t.zero_()
+		t_pre = time.perf_counter()
+		while time.perf_counter() - t_pre < 0.3:
+			for _ in range(5):
+				step()
+			torch.cuda.synchronize()
+		t0 = time.perf_counter()
+		for _ in range(args.steps):
+			step()
+		torch.cuda.synchronize()
+		ms0 = (time.perf_counter() - t0) * 1e3 / args.steps
+		out["zero_operands"] = {"ms_per_step": ms0, "speedup_over_timed_run": ms / ms0,
+		                        "what": "same launches, q = k = v = dO = 0 (identical instruction stream and traffic)"}
 	if not args.no_mfma_peak:
 		mp = mfma_peak(torch, dev)
 		out["mfma_peak_measured"] = mp
