@@ -1235,7 +1235,7 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 	}
 	auto launch_dq = [&]() {
 		a.mtiles = (a.Sq + C::DQ_BM - 1) / C::DQ_BM;
-		a.interleave = a.xcd_remap == 1 ? launch_order(a, a.Hq / a.Hkv, groups / 8) : 1;
+		a.interleave = a.xcd_remap == 1 ? launch_order(a, a.Hq / a.Hkv, groups / 8, (int64_t)a.Sk * D * 4) : 1;
 		dim3 grid((unsigned)(a.mtiles * a.B * a.Hq)), block(C::DQ_NW * 64);
 		if (BIAS && a.dbias && a.softcap > 0.f)
 			hipLaunchKernelGGL((bwd_dq_kernel<T, D, C::DQ_NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, false, BIAS, BIAS>), grid, block, 0, s, a);
@@ -1251,7 +1251,7 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 	if (fused_delta) launch_dq();
 	if (a.stages & 2) {
 		a.mtiles = (a.Sk + C::KV_BN - 1) / C::KV_BN;
-		a.interleave = a.xcd_remap == 1 ? launch_order(a, 1, groups / 8) : 1;
+		a.interleave = a.xcd_remap == 1 ? launch_order(a, 1, groups / 8, (int64_t)(a.Hq / a.Hkv) * a.Sq * D * 4) : 1;
 		dim3 grid((unsigned)(a.mtiles * a.B * a.Hkv)), block(C::KV_NW * 64);
 		// typed variant: bias in the element type of q; where it stages the bias through LDS (D <= 128)
 		// it also needs 16-byte aligned rows of whole 16-byte pieces

@@ -40,10 +40,13 @@ constexpr float kFastSum = 16384.f;
 // index, so the launch order makes every aligned run of four workgroups of an XCD the same tile index: of the
 // `heads` equal-length items a group has per tile (r q-heads for the forward and dQ kernels, 1 for dK/dV) and, where
 // those are fewer than four, of `e` groups that advance together.  Returns e (1, 2 or 4); per_xcd = groups per XCD.
-inline int launch_order(const KArgs& a, int heads, int per_xcd) {
+// Groups that advance together also stream their operands together (K and V in the forward and dQ kernels, Q and dO
+// of the group's q-heads in dK/dV: stream_bytes per group): e is kept small enough for these to stay within reach of
+// the XCD's 4 MiB L2 - with four groups of 8 MiB each the dK/dV kernel fetched twice as much from memory for no gain.
+inline int launch_order(const KArgs& a, int heads, int per_xcd, int64_t stream_bytes) {
 	if (a.win_right < 0 && a.win_left < 0) return 1;  // every tile sees all keys: equal lengths anyway
 	int e = heads % 4 == 0 ? 1 : (heads % 2 == 0 ? 2 : 4);
-	while (e > 1 && per_xcd % e) e >>= 1;
+	while (e > 1 && (per_xcd % e || e * stream_bytes > (8 << 20))) e >>= 1;
 	return e;
 }
 
@@ -841,7 +844,7 @@ hipError_t launch_fwd_t(bool bias, bool drop, KArgs& a, hipStream_t s) {
 	a.mtiles = (a.Sq + C::BM - 1) / C::BM;
 	int groups = a.B * a.Hkv;
 	a.xcd_remap = (groups % 8 == 0) ? 1 : 0;
-	a.interleave = a.xcd_remap ? launch_order(a, a.Hq / a.Hkv, groups / 8) : 1;
+	a.interleave = a.xcd_remap ? launch_order(a, a.Hq / a.Hkv, groups / 8, (int64_t)a.Sk * D * 4) : 1;
 	if (bias && a.bias_sh == 0 && a.B % 8 == 0) a.xcd_remap = a.kv_lens ? 3 : 2;
 	dim3 grid((unsigned)(a.mtiles * a.B * a.Hq)), block(C::NW * 64);
 	const bool blds = bias && a.bias_lds && D <= 128;
