@@ -24,6 +24,13 @@ forgets what is pending at an unconditional branch; a v_mfma between `;;#ASMSTAR
       spill off (-mllvm -amdgpu-spill-vgpr-to-agpr=0); this rule is the check that no operand is left
       partly unwritten.  (Other instructions are not checked: under a divergent branch the compiler
       legitimately reads registers that are only written for the lanes that use them.)
+  R4  (loops that stream tiles: blocks the compiler marks `Depth=2` or deeper) no access to scratch memory, and no
+      `s_waitcnt vmcnt` that a matrix product follows in the same block - unless the block itself loads values from
+      global memory into registers (the variants that read bias or mask values one by one).  The counter behind
+      vmcnt also counts the direct-to-LDS copies of the next tile, which are issued at the start of a step: a spill
+      reload or a late wait for a value loaded before the loop makes every step wait for those copies.
+      A violation fails the build for the kernel variants without bias and without dropout (the first two boolean
+      template arguments); for the other variants, whose register budget is tighter, it is printed as a note.
 A wait state is one instruction; `s_nop N` counts N + 1.
 
 Usage: asm_lint.py FILE.s [FILE.s ...]   (exit status 1 and one line per violation)
@@ -141,6 +148,59 @@ def lint(path: str):
 				dst, c = _regs(ops[0]), _regs(ops[3])
 				pending.append({"line": ln, "c": (c if c and c != dst else None), "dst": dst, "mfma": 0, "wait": 0})
 	return problems
+
+
+_DEPTH = re.compile(r"^(\.L[\w$]+):.*Depth=(\d+)")
+
+
+def lint_loops(path: str):
+	"""Rule R4: nothing in a tile loop waits on the memory counter that the tile copies share."""
+	problems, notes = [], []
+	kernel = "?"
+	blocks = []  # (label, depth, [(ln, text)])
+	cur = None
+
+	def flush():
+		flags = re.findall(r"Lb([01])E", kernel)[:2]
+		strict = flags == ["0", "0"]
+		out = problems if strict else notes
+		# variants that read bias or mask values one by one load into registers inside the loops: their waits are their own
+		loads = any(t.startswith(("global_load_", "buffer_load_", "flat_load_")) and not t.startswith("global_load_lds")
+		            for _, depth, insts in blocks if depth >= 2 for _, t in insts)
+		for label, depth, insts in blocks:
+			if depth < 2 or loads:
+				continue
+			for i, (ln, t) in enumerate(insts):
+				if t.startswith(("scratch_load", "scratch_store")):
+					out.append(f"{path}:{ln}: {kernel}: R4: scratch access `{t.split(';')[0].strip()}` inside a tile loop ({label})")
+				elif t.startswith("s_waitcnt") and "vmcnt" in t:
+					if any(u.startswith("v_mfma") for _, u in insts[i + 1:]):
+						out.append(f"{path}:{ln}: {kernel}: R4: `{t}` ahead of matrix products inside a tile loop ({label})")
+
+	with open(path) as f:
+		for ln, raw in enumerate(f, 1):
+			s = raw.strip()
+			m = _LABEL.match(s)
+			if m:
+				flush()
+				kernel, blocks, cur = m.group(1), [], None
+				continue
+			if s.startswith(".Lfunc_end"):
+				flush()
+				blocks, cur = [], None
+				continue
+			md = _DEPTH.match(s)
+			if md:
+				cur = (md.group(1), int(md.group(2)), [])
+				blocks.append(cur)
+				continue
+			if _BLOCK.match(s):
+				cur = None  # a block outside any loop
+				continue
+			if cur is not None and s and not s.startswith((";", ".")):
+				cur[2].append((ln, s))
+	flush()
+	return problems, notes
 
 
 _TARGET = re.compile(r"^(s_cbranch_\w+|s_branch)\s+(\S+)")
@@ -262,6 +322,10 @@ def main(argv):
 	for path in argv[1:]:
 		bad += lint(path)
 		bad += lint_defined(path)
+		p4, n4 = lint_loops(path)
+		bad += p4
+		for n in n4:
+			print("note: " + n)
 	for b in bad:
 		print(b)
 	if bad:
