@@ -268,11 +268,14 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		return x;
 	};
 	// lse in the units the elementwise stage wants, both negated where they start the chains
-	const float stat_mul = (tid < BMQ ? (FOLD ? inv_scale : (BIAS ? 1.f : kLog2e)) : 1.f) * (FOLD ? -1.f : 1.f);
+	// (lse: -lse / (scale log2(e)) ... in the units of the raw dot product where it starts the chain of S, else -lse log2(e),
+	// the addend of the fused multiply-add that forms the exponent; delta: negated where it starts the chain of dP)
+	const float stat_mul = tid < BMQ ? (FOLD ? -inv_scale : -kLog2e) : (FOLD ? -1.f : 1.f);
 	auto store_stat = [&](float x, int buf) {
 		if (tid < 2 * BMQ) {
 			int which = tid / BMQ;
-			*(FA2_LDS float*)(stat + (2 * which + buf) * STAT_BYTES + stat_row * 4) = x * stat_mul;
+			// (kept finite: lse of a row whose keys all carry the finfo.min "mask" bias of the bf16 type is -3.39e38)
+			*(FA2_LDS float*)(stat + (2 * which + buf) * STAT_BYTES + stat_row * 4) = __builtin_fminf(x * stat_mul, 3.0e38f);
 		}
 	};
 
@@ -376,10 +379,10 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 				if (CAP && a.bias == nullptr)
 					bv[qb & 1][i] = 0.f;
 				else if constexpr (BIAS_T)
-					bv[qb & 1][i] = (float)*(const typename T::E*)pp;
+					bv[qb & 1][i] = to_f32(*(const typename T::E*)pp);
 				else
 					bv[qb & 1][i] = a.bias_dtype == 3   ? *(const float*)pp
-					                : a.bias_dtype == 2 ? (float)*(const __bf16*)pp
+					                : a.bias_dtype == 2 ? to_f32(*(const __bf16*)pp)
 					                : a.bias_dtype == 1 ? (float)*(const _Float16*)pp
 					                                    : (*(const uint8_t*)pp ? 0.f : a.mask_fill);
 			}
@@ -527,16 +530,16 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 					int i = 4 * q + e;
 					if constexpr (BIAS)
 						if constexpr (BIAS_LDS) {
-							float bvl = (float)__builtin_bit_cast(typename T::V4, bvr[qb & 1][q])[e];
-							bx[q][e] = (__builtin_fmaf(sa[i], c1, bvl) - lse4[q][e]) * kLog2e;
+							float bvl = to_f32x4(__builtin_bit_cast(typename T::V4, bvr[qb & 1][q]))[e];
+							bx[q][e] = __builtin_fmaf(__builtin_fmaf(sa[i], c1, bvl), kLog2e, lse4[q][e]);
 						} else if constexpr (CAP) {
 							bt[q][e] = tanh_fast(sa[i] * a.cap_k1);
-							bx[q][e] = (__builtin_fmaf(bt[q][e], a.softcap, bv[qb & 1][i]) - lse4[q][e]) * kLog2e;
+							bx[q][e] = __builtin_fmaf(__builtin_fmaf(bt[q][e], a.softcap, bv[qb & 1][i]), kLog2e, lse4[q][e]);
 						} else {
-							bx[q][e] = (__builtin_fmaf(sa[i], c1, bv[qb & 1][i]) - lse4[q][e]) * kLog2e;
+							bx[q][e] = __builtin_fmaf(__builtin_fmaf(sa[i], c1, bv[qb & 1][i]), kLog2e, lse4[q][e]);
 						}
 					else
-						bx[q][e] = __builtin_fmaf(sa[i], c1, -lse4[q][e]);
+						bx[q][e] = __builtin_fmaf(sa[i], c1, lse4[q][e]);
 				}
 			} else if (phase == 1) {
 #pragma unroll
@@ -882,7 +885,9 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 		int64_t idx = ((int64_t)b * a.Hq + h) * a.Sq + ic;
 		float l = a.lse[idx];
 		// rows without any allowed key carry lse = -inf; their P is forced to 0 by the mask
-		lse_r[qb] = BIAS ? l : l * kLog2e;
+		// the addend of the fused multiply-add that forms the exponent, (x - lse) log2(e) = x log2(e) - lse log2(e); kept finite
+		// for a row whose keys all carry the finfo.min "mask" bias of the bf16 type (lse = -3.39e38: its P underflows to 0)
+		lse_r[qb] = __builtin_fminf(-l * kLog2e, 3.0e38f);
 		del_r[qb] = a.delta[idx];
 	}
 	int wave_jmin, wave_jmax, wave_lmin = kNoKey, wave_lmax = kNoKey;
@@ -1088,11 +1093,11 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 						float p, th = 0.f;
 						if constexpr (CAP) {
 							th = tanh_fast(s[qb][i] * a.cap_k1);
-							p = exp2_fast((__builtin_fmaf(th, a.softcap, bv[qb][aa][e]) - lse_r[qb]) * kLog2e);
+							p = exp2_fast(__builtin_fmaf(__builtin_fmaf(th, a.softcap, bv[qb][aa][e]), kLog2e, lse_r[qb]));
 						} else if constexpr (BIAS)
-							p = exp2_fast((__builtin_fmaf(s[qb][i], c1, BIAS_LDS ? (float)bvl[aa][e] : bv[qb][aa][e]) - lse_r[qb]) * kLog2e);
+							p = exp2_fast(__builtin_fmaf(__builtin_fmaf(s[qb][i], c1, BIAS_LDS ? to_f32x4(bvl[aa])[e] : bv[qb][aa][e]), kLog2e, lse_r[qb]));
 						else
-							p = exp2_fast(__builtin_fmaf(s[qb][i], c1, -lse_r[qb]));
+							p = exp2_fast(__builtin_fmaf(s[qb][i], c1, lse_r[qb]));
 						if constexpr (MASKED) {
 							int j = n0 + 32 * kb + 8 * aa + 4 * g + e;
 							p = ((j <= jmax[qb]) & (j >= jmin[qb])) ? p : 0.f;

@@ -115,6 +115,19 @@ FA2_DEV typename T::V8 pack8(float x0, float x1, float x2, float x3, float x4, f
 	return __builtin_bit_cast(typename T::V8, u);
 }
 
+// 16-bit element -> fp32.  A bf16 value is the upper half of the fp32 with the same value; written as the shift itself
+// because the compiler's extension adds a multiply by 1.0 (it quiets signalling NaNs), one more vector-ALU instruction per
+// bias value in loops that are bound by exactly those.
+FA2_DEV float to_f32(__bf16 x) { return __builtin_bit_cast(float, (uint32_t)__builtin_bit_cast(uint16_t, x) << 16); }
+FA2_DEV float to_f32(_Float16 x) { return (float)x; }
+FA2_DEV f32x4 to_f32x4(bf16x4 x) {
+	u32x2 u = __builtin_bit_cast(u32x2, x);
+	f32x4 r = {__builtin_bit_cast(float, u[0] << 16), __builtin_bit_cast(float, u[0] & 0xffff0000u), __builtin_bit_cast(float, u[1] << 16),
+	           __builtin_bit_cast(float, u[1] & 0xffff0000u)};
+	return r;
+}
+FA2_DEV f32x4 to_f32x4(f16x4 x) { return __builtin_convertvector(x, f32x4); }
+
 FA2_DEV float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
 FA2_DEV float log2_fast(float x) { return __builtin_amdgcn_logf(x); }
 // tanh(x) = 1 - 2 / (1 + e^(2x)): one exp2, one reciprocal; exactly +-1 at the ends of the range

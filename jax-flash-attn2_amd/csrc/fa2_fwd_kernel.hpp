@@ -105,7 +105,7 @@ FA2_DEV f32x4 load_bias4(const char* rowp, int col, int dtype, bool vec_ok, int 
 			out = *(const f32x4*)(rowp + (int64_t)col * 4);
 		} else if (dtype == 2) {
 			bf16x4 t = *(const bf16x4*)(rowp + (int64_t)col * 2);
-			out = __builtin_convertvector(t, f32x4);
+			out = to_f32x4(t);
 		} else if (dtype == 1) {
 			f16x4 t = *(const f16x4*)(rowp + (int64_t)col * 2);
 			out = __builtin_convertvector(t, f32x4);
@@ -122,7 +122,7 @@ FA2_DEV f32x4 load_bias4(const char* rowp, int col, int dtype, bool vec_ok, int 
 				if (dtype == 3)
 					x = *(const float*)(rowp + (int64_t)(col + e) * 4);
 				else if (dtype == 2)
-					x = (float)*(const __bf16*)(rowp + (int64_t)(col + e) * 2);
+					x = to_f32(*(const __bf16*)(rowp + (int64_t)(col + e) * 2));
 				else if (dtype == 1)
 					x = (float)*(const _Float16*)(rowp + (int64_t)(col + e) * 2);
 				else
@@ -403,7 +403,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 #pragma unroll
 				for (int aa = 0; aa < 4; ++aa) {
 					typename T::V4 x = *(const FA2_LDS typename T::V4*)(lds + 4 * TILE_BYTES + boff_lane + (((kb * 4 + aa) << 4) ^ bkey16));
-					bv[kb][0][aa] = __builtin_convertvector(x, f32x4);
+					bv[kb][0][aa] = to_f32x4(x);
 				}
 		} else if constexpr (BIAS) {
 #pragma unroll
@@ -628,14 +628,29 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 						for (int i = 0; i < 16; ++i) oacc[qb][db][i] *= alpha;
 				}
 				const float m_use = mrow[qb] == -INFINITY ? 0.f : mrow[qb];
+				// (x - m) log2(e) as one fused multiply-add, x log2(e) - m log2(e) - unless some row's reference is so
+				// large that m log2(e) leaves the fp32 range: a row whose keys all carry the finfo.min "mask" bias of
+				// the bf16 type (-3.39e38).  Such a wave (rare) subtracts first.
+				if (__builtin_amdgcn_ballot_w64(__builtin_fabsf(m_use) > 1e37f) == 0) {
+					const float nm2 = -m_use * kLog2e;
 #pragma unroll
-				for (int kb = 0; kb < KB; ++kb)
+					for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-					for (int i = 0; i < 16; ++i) {
-						float p = exp2_fast(__builtin_fmaf(s[kb][qb][i] - m_use, kLog2e, 0.f));
-						ls4[i & 3] += p;
-						s[kb][qb][i] = p;
-					}
+						for (int i = 0; i < 16; ++i) {
+							float p = exp2_fast(__builtin_fmaf(s[kb][qb][i], kLog2e, nm2));
+							ls4[i & 3] += p;
+							s[kb][qb][i] = p;
+						}
+				} else {
+#pragma unroll
+					for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+						for (int i = 0; i < 16; ++i) {
+							float p = exp2_fast((s[kb][qb][i] - m_use) * kLog2e);
+							ls4[i & 3] += p;
+							s[kb][qb][i] = p;
+						}
+				}
 				lrow[qb] += (ls4[0] + ls4[1]) + (ls4[2] + ls4[3]);
 				pack_p(qb);
 			}
