@@ -200,7 +200,11 @@ int fa2_bwd_static(const fa2_params* p, void* hip_stream);
 
 /* keep[b,h,i,j] (uint8, contiguous [B,Hq,Sq,Sk]) of the dropout mask the
  * kernels apply for (seed, p_drop); for validation against the Philox
- * definition.  Counterpart of `tl.rand(seed, offs) > p`
+ * definition: Philox-4x32-10 with key (seed low word, seed high word), one call per
+ * two adjacent rows x four adjacent keys with counter (j >> 2, i >> 1, h, b); its four
+ * words are eight 16-bit values (word w: value 2w in the low half, 2w + 1 in the high
+ * half), element (i, j) owns value 4 (i & 1) + (j & 3) and is kept iff
+ * value >= floor(p_drop * 65536).  Counterpart of `tl.rand(seed, offs) > p`
  * (_forward_triton.py:140-143). Uses B, Hq, Sq, Sk, p_drop, seed / seed_dev only. */
 int fa2_dropout_mask(const fa2_params* p, uint8_t* keep, void* hip_stream);
 
