@@ -380,6 +380,17 @@ FA2_DEV void philox4x32_rounds(uint32_t (&c)[4], uint32_t k0, uint32_t k1) {
 // value `half` (0 / 1) of a word against the threshold
 FA2_DEV bool keep16(uint32_t word, int half, uint32_t thr16) { return (half ? (word >> 16) : (word & 0xffffu)) >= thr16; }
 
+// Two packed 16-bit elements `x` against the two 16-bit values of `word` (low half with low half): an element whose value is
+// below the threshold becomes +0.  thr2 = the threshold in both halves.  Three packed 16-bit integer operations:
+// d = thr -sat value is non-zero exactly for a dropped element, 1 -sat d is the factor 1 / 0.
+FA2_DEV uint32_t keep_pair16(uint32_t x, uint32_t word, uint32_t thr2) {
+	typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+	const u16x2 one = {1, 1};
+	u16x2 d = __builtin_elementwise_sub_sat(__builtin_bit_cast(u16x2, thr2), __builtin_bit_cast(u16x2, word));
+	u16x2 k = __builtin_elementwise_sub_sat(one, d);
+	return __builtin_bit_cast(uint32_t, (u16x2)(__builtin_bit_cast(u16x2, x) * k));
+}
+
 // the neighbouring lane's value (lanes 0 <-> 1, 2 <-> 3 of every quad)
 FA2_DEV uint32_t quad_swap1(uint32_t x) { return (uint32_t)__builtin_amdgcn_mov_dpp((int)x, 0xB1, 0xf, 0xf, false); }
 
@@ -388,28 +399,38 @@ FA2_DEV uint32_t quad_swap1(uint32_t x) { return (uint32_t)__builtin_amdgcn_mov_
 // the row's four values for keys jb + 8 aa .. + 3.  SHARE: the lane of the even row evaluates the calls of aa = 0, 2,
 // the lane of the odd row those of aa = 1, 3, and they exchange (needs lane ^ 1 = row ^ 1 in the same (b, h));
 // otherwise every lane evaluates its four calls itself.
+// One half of that: the words of aa = 2 pr and 2 pr + 1 (with SHARE one generator call per lane).
 template <bool SHARE>
-FA2_DEV void dropout_words_rowlane(int jb, uint32_t row, uint32_t h, uint32_t b, uint32_t k0, uint32_t k1, uint32_t (&w)[4][2]) {
+FA2_DEV void dropout_words_rowlane_half(int jb, uint32_t row, uint32_t h, uint32_t b, uint32_t k0, uint32_t k1, int pr, uint32_t (&w)[2][2]) {
 	const bool odd = row & 1u;
 	if constexpr (SHARE) {
-#pragma unroll
-		for (int pr = 0; pr < 2; ++pr) {
-			int aa_mine = 2 * pr + (odd ? 1 : 0);
-			u32x4 r = philox4x32_10((uint32_t)((jb + 8 * aa_mine) >> 2), row >> 1, h, b, k0, k1);
-			uint32_t own0 = odd ? r[2] : r[0], own1 = odd ? r[3] : r[1];
-			uint32_t got0 = quad_swap1(odd ? r[0] : r[2]), got1 = quad_swap1(odd ? r[1] : r[3]);
-			w[2 * pr][0] = odd ? got0 : own0;
-			w[2 * pr][1] = odd ? got1 : own1;
-			w[2 * pr + 1][0] = odd ? own0 : got0;
-			w[2 * pr + 1][1] = odd ? own1 : got1;
-		}
+		int aa_mine = 2 * pr + (odd ? 1 : 0);
+		u32x4 r = philox4x32_10((uint32_t)((jb + 8 * aa_mine) >> 2), row >> 1, h, b, k0, k1);
+		uint32_t own0 = odd ? r[2] : r[0], own1 = odd ? r[3] : r[1];
+		uint32_t got0 = quad_swap1(odd ? r[0] : r[2]), got1 = quad_swap1(odd ? r[1] : r[3]);
+		w[0][0] = odd ? got0 : own0;
+		w[0][1] = odd ? got1 : own1;
+		w[1][0] = odd ? own0 : got0;
+		w[1][1] = odd ? own1 : got1;
 	} else {
 #pragma unroll
-		for (int aa = 0; aa < 4; ++aa) {
-			u32x4 r = philox4x32_10((uint32_t)((jb + 8 * aa) >> 2), row >> 1, h, b, k0, k1);
-			w[aa][0] = odd ? r[2] : r[0];
-			w[aa][1] = odd ? r[3] : r[1];
+		for (int u = 0; u < 2; ++u) {
+			u32x4 r = philox4x32_10((uint32_t)((jb + 8 * (2 * pr + u)) >> 2), row >> 1, h, b, k0, k1);
+			w[u][0] = odd ? r[2] : r[0];
+			w[u][1] = odd ? r[3] : r[1];
 		}
+	}
+}
+template <bool SHARE>
+FA2_DEV void dropout_words_rowlane(int jb, uint32_t row, uint32_t h, uint32_t b, uint32_t k0, uint32_t k1, uint32_t (&w)[4][2]) {
+#pragma unroll
+	for (int pr = 0; pr < 2; ++pr) {
+		uint32_t half[2][2];
+		dropout_words_rowlane_half<SHARE>(jb, row, h, b, k0, k1, pr, half);
+		w[2 * pr][0] = half[0][0];
+		w[2 * pr][1] = half[0][1];
+		w[2 * pr + 1][0] = half[1][0];
+		w[2 * pr + 1][1] = half[1][1];
 	}
 }
 

@@ -476,21 +476,8 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 		V8 pf[QB][BN / 16];
 		compute_s();
 		issue_v(std::integral_constant<int, 0>{}, vfr[0]);
-		// packs P (held in s) to the B operand of the second product, after dropout
+		// packs P (held in s) to the B operand of the second product
 		auto pack_p = [&](int qb) __attribute__((always_inline)) {
-			if constexpr (DROP) {
-#pragma unroll
-				for (int kb = 0; kb < KB; ++kb) {
-					uint32_t dw[4][2];
-					// (split forward: the rows of a tile may belong to several heads - no sharing between lanes)
-					dropout_words_rowlane<!SPLIT>(n0 + 32 * kb + 4 * g, (uint32_t)qrow[qb], (uint32_t)hl[qb], (uint32_t)b, drop_k0, drop_k1, dw);
-#pragma unroll
-					for (int aa = 0; aa < 4; ++aa)
-#pragma unroll
-						for (int e = 0; e < 4; ++e)
-							s[kb][qb][4 * aa + e] = keep16(dw[aa][e >> 1], e & 1, a.drop_thr) ? s[kb][qb][4 * aa + e] : 0.f;
-				}
-			}
 #pragma unroll
 			for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
@@ -500,14 +487,34 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 					                               r[8 * hf + 5], r[8 * hf + 6], r[8 * hf + 7]);
 				}
 		};
+		// Dropout on the packed P (the row sums have been taken before): word m of a packed operand holds the keys
+		// 8 (2 hf + m / 2) + 4 g + 2 (m % 2), + 1 of the block - the two values of word m % 2 of the generator's words for that
+		// group of four keys.
+		// (split forward: the rows of a tile may belong to several heads - no sharing of generator calls between lanes)
+		auto drop_p = [&](int qb) __attribute__((always_inline)) {
+			if constexpr (DROP) {
+				const uint32_t thr2 = a.drop_thr * 0x10001u;
+#pragma unroll
+				for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+					for (int hf = 0; hf < 2; ++hf) {
+						uint32_t dw[2][2];
+						dropout_words_rowlane_half<!SPLIT>(n0 + 32 * kb + 4 * g, (uint32_t)qrow[qb], (uint32_t)hl[qb], (uint32_t)b, drop_k0, drop_k1, hf, dw);
+						u32x4 x = __builtin_bit_cast(u32x4, pf[qb][2 * kb + hf]);
+#pragma unroll
+						for (int m = 0; m < 4; ++m) x[m] = keep_pair16(x[m], dw[m >> 1][m & 1], thr2);
+						pf[qb][2 * kb + hf] = __builtin_bit_cast(V8, x);
+					}
+			}
+		};
 		if constexpr (FOLD) {
-			// Fast path (not with dropout): P = exp2(c1 S - c1 m) against the reference m the rows
+			// Fast path: P = exp2(c1 S - c1 m) against the reference m the rows
 			// already have, packed to 16 bits at once - no row maximum, and the scores stay in their
 			// registers.  It stands when every partial row sum of the tile stays below kFastSum (then no
 			// P exceeds it either: 16-bit P and the fp32 sums hold that without loss) and no row meets
 			// its first keys in this tile.  Otherwise (decided for the wave as a whole) the tile takes
 			// the path with the row maximum, from the scores that are still there.
-			constexpr bool FAST = !DROP;
+			constexpr bool FAST = true;
 			float lt[QB];
 			bool slow = true;
 			if constexpr (FAST) {
@@ -655,6 +662,8 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 				pack_p(qb);
 			}
 		}
+#pragma unroll
+		for (int qb = 0; qb < QB; ++qb) drop_p(qb);
 
 		// O^T += V^T P^T
 		auto pv_batch = [&](auto batch_tag) {
