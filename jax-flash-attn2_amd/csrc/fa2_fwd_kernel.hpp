@@ -690,6 +690,182 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 		__builtin_amdgcn_sched_barrier(0);
 	};
 
+	// Head dim 256 runs one wave per SIMD, so the softmax overlaps the matrix products only if the wave interleaves
+	// them itself.  A tile without masking is handled as two halves of 32 keys, in four phases of KS products each:
+	//   phase 0   S_0 = K_0 Q^T         |  (dropout: the generator calls of half 0)
+	//   phase 1   S_1 = K_1 Q^T         |  P_0 from S_0   (dropout: mask on P_0, first rounds of the calls of half 1)
+	//   phase 2   O^T += V_0^T P_0^T    |  P_1 from S_1   (dropout: their last rounds, mask on P_1)
+	//   phase 3   O^T += V_1^T P_1^T
+	// The vector-ALU work is cut into pieces that follow the products one by one, and every product is preceded by the
+	// LDS read of a fragment PA products further on (a scheduling barrier after every slot pins that order).  The
+	// softmax is the path without the row maximum, applied per half; a half that needs the maximum after all (decided
+	// for the wave as a whole) takes it from its scores, which are still in their registers, before its P is used.
+	constexpr bool PIPE = D == 256 && NW == 4 && QB == 1 && FOLD && !SPLIT;
+	auto tile_pipe = [&](int n0) {
+		if constexpr (PIPE) {
+			constexpr int NFR = KS;  // fragments = products of a phase: KS of K for a half, 2 sixteen-key steps x DB of V
+			constexpr int RING = 8, PA = DROP ? 4 : 7;  // (dropout: the generator needs the registers)
+			static_assert(2 * DB == KS && KS % RING == 0 && PA < RING, "");
+			u32x4 fr[RING];
+			f32x16 sc[2];
+			u32x4 pp[2][2];  // [half][16-key step]: P packed to 16 bits
+			float bx[4], lsum[4];
+			auto read_k = [&](int hf, int f) __attribute__((always_inline)) {
+				fr[f % RING] = __builtin_bit_cast(u32x4, *(const FA2_LDS V8*)(lds + koff[f % KR] + (f / KR) * 256 + hf * (32 * D * 2)));
+			};
+			auto read_v = [&](int hf, int f) __attribute__((always_inline)) {
+				const int db = f % DB;
+				fr[f % RING] = lds_tr_issue_rt<D>(lds + voff[db % DR][0] + (db / DR) * 256, lds + voff[db % DR][1] + (db / DR) * 256, 2 * hf + f / DB);
+			};
+			auto prod_s = [&](int hf, int f) __attribute__((always_inline)) {
+				f32x16 zero;
+#pragma unroll
+				for (int i = 0; i < 16; ++i) zero[i] = 0.f;
+				sc[hf] = mfma32(as_frag<T>(fr[f % RING]), qf[0][f], f == 0 ? zero : sc[hf]);
+			};
+			auto prod_o = [&](int hf, int f) __attribute__((always_inline)) {
+				oacc[0][f % DB] = mfma32(as_frag<T>(fr[f % RING]), as_frag<T>(pp[hf][f / DB]), oacc[0][f % DB]);
+			};
+			// piece pc (0 .. 7) of the softmax of a half: values 4 q .. 4 q + 3 (q = pc / 2); first the exponents and two
+			// exp2, then two exp2, the sums and the packing - a result is consumed some instructions after it was produced
+			auto soft_piece = [&](int hf, int pc) __attribute__((always_inline)) {
+				const int q = pc >> 1;
+				if ((pc & 1) == 0) {
+#pragma unroll
+					for (int e = 0; e < 4; ++e) bx[e] = __builtin_fmaf(sc[hf][4 * q + e], c1, nmc[0]);
+					bx[0] = exp2_fast(bx[0]);
+					bx[1] = exp2_fast(bx[1]);
+				} else {
+					bx[2] = exp2_fast(bx[2]);
+					bx[3] = exp2_fast(bx[3]);
+#pragma unroll
+					for (int e = 0; e < 4; ++e) lsum[e] = q == 0 ? bx[e] : lsum[e] + bx[e];
+					pp[hf][q >> 1][2 * (q & 1)] = pack2<typename T::V2>(bx[0], bx[1]);
+					pp[hf][q >> 1][2 * (q & 1) + 1] = pack2<typename T::V2>(bx[2], bx[3]);
+				}
+			};
+			// after the pieces of a half: does the path without the maximum stand?  Otherwise the half is done again
+			// from its scores with the row maximum (raising the reference and rescaling l and O where it exceeds it).
+			auto soft_finish = [&](int hf) __attribute__((always_inline)) {
+				float lt = (lsum[0] + lsum[1]) + (lsum[2] + lsum[3]);
+				// (a NaN sum - from inf or NaN inputs - also takes the other path, which propagates it)
+				const bool over = !(lt <= kFastSum) || mrow[0] == -INFINITY;
+				if (__builtin_amdgcn_ballot_w64(over) != 0) {
+					float mx4[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+#pragma unroll
+					for (int i = 0; i < 16; ++i) mx4[i & 3] = __builtin_fmaxf(mx4[i & 3], sc[hf][i]);
+					float mx = pair_max(__builtin_fmaxf(__builtin_fmaxf(mx4[0], mx4[1]), __builtin_fmaxf(mx4[2], mx4[3])));
+					if (mx > mrow[0]) {
+						const float alpha = exp2_fast((mrow[0] - mx) * c1);
+						mrow[0] = mx;
+						nmc[0] = -mx * c1;
+						lrow[0] *= alpha;
+#pragma unroll
+						for (int db = 0; db < DB; ++db)
+#pragma unroll
+							for (int i = 0; i < 16; ++i) oacc[0][db][i] *= alpha;
+					}
+					float ls4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+					for (int i = 0; i < 16; ++i) {
+						float pv = exp2_fast(__builtin_fmaf(sc[hf][i], c1, nmc[0]));
+						ls4[i & 3] += pv;
+						sc[hf][i] = pv;
+					}
+#pragma unroll
+					for (int h2 = 0; h2 < 2; ++h2)
+						pp[hf][h2] = __builtin_bit_cast(u32x4, pack8<T>(sc[hf][8 * h2 + 0], sc[hf][8 * h2 + 1], sc[hf][8 * h2 + 2], sc[hf][8 * h2 + 3],
+						                                                  sc[hf][8 * h2 + 4], sc[hf][8 * h2 + 5], sc[hf][8 * h2 + 6], sc[hf][8 * h2 + 7]));
+					lt = (ls4[0] + ls4[1]) + (ls4[2] + ls4[3]);
+				}
+				lrow[0] += lt;
+			};
+			// Dropout: the two generator calls of a half (one per 16-key step; see dropout_words_rowlane_half), one after the
+			// other, as pieces of two rounds each, and the mask on the packed P (see drop_p in the other tile body).
+			uint32_t cs[4], dwp[2][2][2][2];  // state of the call in flight; words [half][call][group of four keys][word]
+			const bool odd = qrow[0] & 1;
+			const uint32_t thr2 = a.drop_thr * 0x10001u;
+			// piece pc of call u of half hf: 0 .. 4 = rounds 2 pc, 2 pc + 1 (the counter is set up with the first), 5 = exchange
+			auto gen_piece = [&](int hf, int u, auto pt) __attribute__((always_inline)) {
+				if constexpr (DROP) {
+					constexpr int pc = decltype(pt)::value;
+					if constexpr (pc == 0) {
+						cs[0] = (uint32_t)((n0 + 32 * hf + 4 * g + 8 * (2 * u + (odd ? 1 : 0))) >> 2);
+						cs[1] = (uint32_t)qrow[0] >> 1;
+						cs[2] = (uint32_t)hl[0];
+						cs[3] = (uint32_t)b;
+					}
+					if constexpr (pc < 5) {
+						philox4x32_rounds<2 * pc, 2 * pc + 2>(cs, drop_k0, drop_k1);
+					} else {
+						uint32_t own0 = odd ? cs[2] : cs[0], own1 = odd ? cs[3] : cs[1];
+						uint32_t got0 = quad_swap1(odd ? cs[0] : cs[2]), got1 = quad_swap1(odd ? cs[1] : cs[3]);
+						dwp[hf][u][0][0] = odd ? got0 : own0;
+						dwp[hf][u][0][1] = odd ? got1 : own1;
+						dwp[hf][u][1][0] = odd ? own0 : got0;
+						dwp[hf][u][1][1] = odd ? own1 : got1;
+					}
+				}
+			};
+			auto mask_piece = [&](int hf, int u) __attribute__((always_inline)) {
+				if constexpr (DROP) {
+#pragma unroll
+					for (int m = 0; m < 4; ++m) pp[hf][u][m] = keep_pair16(pp[hf][u][m], dwp[hf][u][m >> 1][m & 1], thr2);
+				}
+			};
+			// one phase: NFR slots of (read ahead, product, vector-ALU piece)
+			auto phase = [&](auto&& read_cur, auto&& prod, auto&& read_next, auto&& valu) __attribute__((always_inline)) {
+				__builtin_amdgcn_sched_barrier(0);
+				static_for<0, NFR>([&](auto jt) __attribute__((always_inline)) {
+					constexpr int j = decltype(jt)::value;
+					if constexpr (j + PA < NFR)
+						read_cur(j + PA);
+					else
+						read_next(j + PA - NFR);
+					prod(j);
+					__builtin_amdgcn_sched_barrier(0);
+					valu(jt);
+					__builtin_amdgcn_sched_barrier(0);
+				});
+			};
+			auto none = [&](auto) __attribute__((always_inline)) {};
+			// the eight pieces of a half follow the products 2 .. 9 of the phase (the scores' last product is then at
+			// least two products back)
+			// (dropout: both calls of half 0 run in phase 0, the first call of half 1 at the end of phase 1, its second at the end of phase 2;
+			// the mask of a half is applied once its P is final: after soft_finish, before the phase that uses it)
+			auto gv0 = [&](auto jt) __attribute__((always_inline)) {
+				constexpr int j = decltype(jt)::value;
+				if constexpr (j < 12) gen_piece(0, j / 6, std::integral_constant<int, j % 6>{});
+			};
+			auto sv0 = [&](auto jt) __attribute__((always_inline)) {
+				constexpr int j = decltype(jt)::value;
+				if constexpr (j >= 2 && j < 10) soft_piece(0, j - 2);
+				if constexpr (j >= 10) gen_piece(1, 0, std::integral_constant<int, j - 10>{});
+			};
+			auto sv1 = [&](auto jt) __attribute__((always_inline)) {
+				constexpr int j = decltype(jt)::value;
+				if constexpr (j >= 2 && j < 10) soft_piece(1, j - 2);
+				if constexpr (j >= 10) gen_piece(1, 1, std::integral_constant<int, j - 10>{});
+			};
+#pragma unroll
+			for (int f = 0; f < PA; ++f) read_k(0, f);
+			phase([&](int f) __attribute__((always_inline)) { read_k(0, f); }, [&](int f) __attribute__((always_inline)) { prod_s(0, f); },
+			      [&](int f) __attribute__((always_inline)) { read_k(1, f); }, gv0);
+			phase([&](int f) __attribute__((always_inline)) { read_k(1, f); }, [&](int f) __attribute__((always_inline)) { prod_s(1, f); },
+			      [&](int f) __attribute__((always_inline)) { read_v(0, f); }, sv0);
+			soft_finish(0);
+			mask_piece(0, 0);
+			mask_piece(0, 1);
+			phase([&](int f) __attribute__((always_inline)) { read_v(0, f); }, [&](int f) __attribute__((always_inline)) { prod_o(0, f); },
+			      [&](int f) __attribute__((always_inline)) { read_v(1, f); }, sv1);
+			soft_finish(1);
+			mask_piece(1, 0);
+			mask_piece(1, 1);
+			phase([&](int f) __attribute__((always_inline)) { read_v(1, f); }, [&](int f) __attribute__((always_inline)) { prod_o(1, f); }, none, none);
+			__builtin_amdgcn_sched_barrier(0);
+		}
+	};
+
 	// One pipeline step: publish tile t, start the copies of tile t + 1, compute.
 	auto step = [&](auto masked_tag, int t) {
 		const int n0 = t * BN;
@@ -709,7 +885,12 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 		}
 		bool skip = false;
 		if constexpr (decltype(masked_tag)::value) skip = n0 > wave_jmax || n0 + BN - 1 < wave_lmin;  // whole tile masked for this wave (uniform)
-		if (!skip) tile_body(masked_tag, n0);
+		if (!skip) {
+			if constexpr (PIPE && !decltype(masked_tag)::value)
+				tile_pipe(n0);
+			else
+				tile_body(masked_tag, n0);
+		}
 		// the other buffers next time
 #pragma unroll
 		for (int ks = 0; ks < KR; ++ks) koff[ks] ^= TILE_BYTES;
