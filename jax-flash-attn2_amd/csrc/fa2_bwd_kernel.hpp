@@ -1147,6 +1147,138 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 		}
 	};
 
+	// Head dim 256 runs one wave per SIMD, so the elementwise stage overlaps the matrix products only if the wave
+	// interleaves them itself (as the forward kernel does at this head dim).  A tile without masking goes as two halves
+	// of 32 keys through four phases,
+	//   phase 0   S_0 = K_0 Q^T, dP_0 = V_0 dO^T      |  (dropout: the generator calls of half 0)
+	//   phase 1   S_1 = K_1 Q^T, dP_1 = V_1 dO^T      |  dS_0 from S_0, dP_0    (dropout: the calls of half 1)
+	//   phase 2   dQ^T += K_0^T dS_0^T                |  dS_1 from S_1, dP_1
+	//   phase 3   dQ^T += K_1^T dS_1^T
+	// with the vector-ALU work in pieces that follow the products one by one and every product preceded by the LDS read
+	// of a fragment PA products further on (a scheduling barrier after every slot pins the order).
+	constexpr bool PIPE = D == 256 && NW == 4 && QB == 1 && !BIAS && !CAP && !DBIAS;
+	auto tile_pipe = [&](int n0) {
+		if constexpr (PIPE) {
+			constexpr int NA = 2 * KS, NC = 2 * DB;  // products of a phase: S and dP alternating; two 16-key steps x DB
+			constexpr int RING = 8, PA = 7;
+			static_assert(NA % RING == 0 && NC % RING == 0 && PA < RING, "");
+			u32x4 fr[RING];
+			f32x16 sc[2], dpc[2];
+			u32x4 dsp[2][2];  // [half][16-key step]: dS packed to 16 bits
+			float bp[4];
+			// fragment f of phase A: k-step f / 2 of K (even f) or V (odd f); of phase C: 16-key step f / DB, d-block f % DB of K^T
+			auto read_a = [&](int hf, int f) __attribute__((always_inline)) {
+				const int ks = f >> 1;
+				fr[f % RING] = __builtin_bit_cast(u32x4, *(const FA2_LDS V8*)(lds + koff[ks % KR] + (ks / KR) * 256 + ((f & 1) ? 2 * TILE_BYTES : 0) + hf * (32 * D * 2)));
+			};
+			auto read_c = [&](int hf, int f) __attribute__((always_inline)) {
+				const int db = f % DB;
+				const FA2_LDS char* kt = lds + hf * (32 * D * 2);
+				fr[f % RING] = lds_tr_issue_rt<D>(kt + toff[db % DR][0] + (db / DR) * 256, kt + toff[db % DR][1] + (db / DR) * 256, f / DB);
+			};
+			auto prod_a = [&](int hf, int f) __attribute__((always_inline)) {
+				f32x16 zero;
+#pragma unroll
+				for (int i = 0; i < 16; ++i) zero[i] = 0.f;
+				const int ks = f >> 1;
+				if (f & 1)
+					dpc[hf] = mfma32(as_frag<T>(fr[f % RING]), dof[0][ks], ks == 0 ? zero : dpc[hf]);
+				else
+					sc[hf] = mfma32(as_frag<T>(fr[f % RING]), qf[0][ks], ks == 0 ? zero : sc[hf]);
+			};
+			auto prod_c = [&](int hf, int f) __attribute__((always_inline)) {
+				dq[0][f % DB] = mfma32(as_frag<T>(fr[f % RING]), as_frag<T>(dsp[hf][f / DB]), dq[0][f % DB]);
+			};
+			// Dropout: the two generator calls of a half, one after the other, in pieces of two rounds each (see the forward kernel)
+			uint32_t cs[4], dwp[2][2][2][2];  // state of the call in flight; words [half][call][group of four keys][word]
+			const bool odd = qrow[0] & 1;
+			auto gen_piece = [&](int hf, int u, auto pt) __attribute__((always_inline)) {
+				if constexpr (DROP) {
+					constexpr int pc = decltype(pt)::value;  // 0 .. 4: rounds 2 pc, 2 pc + 1; 5: exchange with the neighbouring row's lane
+					if constexpr (pc == 0) {
+						cs[0] = (uint32_t)((n0 + 32 * hf + 4 * g + 8 * (2 * u + (odd ? 1 : 0))) >> 2);
+						cs[1] = (uint32_t)qrow[0] >> 1;
+						cs[2] = (uint32_t)h;
+						cs[3] = (uint32_t)b;
+					}
+					if constexpr (pc < 5) {
+						philox4x32_rounds<2 * pc, 2 * pc + 2>(cs, drop_k0, drop_k1);
+					} else {
+						uint32_t own0 = odd ? cs[2] : cs[0], own1 = odd ? cs[3] : cs[1];
+						uint32_t got0 = quad_swap1(odd ? cs[0] : cs[2]), got1 = quad_swap1(odd ? cs[1] : cs[3]);
+						dwp[hf][u][0][0] = odd ? got0 : own0;
+						dwp[hf][u][0][1] = odd ? got1 : own1;
+						dwp[hf][u][1][0] = odd ? own0 : got0;
+						dwp[hf][u][1][1] = odd ? own1 : got1;
+					}
+				}
+			};
+			// piece pc (0 .. 7) of the elementwise stage of a half: values 4 aa .. 4 aa + 3 (aa = pc / 2); first P, then dS and the packing
+			auto ew_piece = [&](int hf, int pc) __attribute__((always_inline)) {
+				const int aa = pc >> 1;
+				if ((pc & 1) == 0) {
+#pragma unroll
+					for (int e = 0; e < 4; ++e) bp[e] = exp2_fast(__builtin_fmaf(sc[hf][4 * aa + e], c1, lse_r[0]));
+				} else {
+					float ds[4];
+#pragma unroll
+					for (int e = 0; e < 4; ++e) {
+						float dpe = dpc[hf][4 * aa + e];
+						if constexpr (DROP) dpe = keep16(dwp[hf][aa >> 1][aa & 1][e >> 1], e & 1, a.drop_thr) ? dpe * a.drop_inv_keep : 0.f;
+						ds[e] = bp[e] * (dpe - del_r[0]);
+					}
+					dsp[hf][aa >> 1][2 * (aa & 1)] = pack2<typename T::V2>(ds[0], ds[1]);
+					dsp[hf][aa >> 1][2 * (aa & 1) + 1] = pack2<typename T::V2>(ds[2], ds[3]);
+				}
+			};
+			auto phase = [&](auto n_tag, auto&& read_cur, auto&& prod, auto&& read_next, auto&& valu) __attribute__((always_inline)) {
+				constexpr int N = decltype(n_tag)::value;
+				__builtin_amdgcn_sched_barrier(0);
+				static_for<0, N>([&](auto jt) __attribute__((always_inline)) {
+					constexpr int j = decltype(jt)::value;
+					if constexpr (j + PA < N)
+						read_cur(j + PA);
+					else
+						read_next(j + PA - N);
+					prod(j);
+					__builtin_amdgcn_sched_barrier(0);
+					valu(jt);
+					__builtin_amdgcn_sched_barrier(0);
+				});
+			};
+			auto none = [&](auto) __attribute__((always_inline)) {};
+			std::integral_constant<int, NA> na;
+			std::integral_constant<int, NC> nc;
+			// phase 0: both calls of half 0 (6 pieces each)
+			auto v0 = [&](auto jt) __attribute__((always_inline)) {
+				constexpr int j = decltype(jt)::value;
+				if constexpr (j < 12) gen_piece(0, j / 6, std::integral_constant<int, j % 6>{});
+			};
+			// phase 1: the pieces of half 0 after the products 2, 4, .. 16; then both calls of half 1
+			auto v1 = [&](auto jt) __attribute__((always_inline)) {
+				constexpr int j = decltype(jt)::value;
+				if constexpr (j >= 2 && j < 18 && j % 2 == 0) ew_piece(0, (j - 2) / 2);
+				if constexpr (j >= 18 && j < 30) gen_piece(1, (j - 18) / 6, std::integral_constant<int, (j - 18) % 6>{});
+			};
+			// phase 2: the pieces of half 1 after the products 2 .. 9
+			auto v2 = [&](auto jt) __attribute__((always_inline)) {
+				constexpr int j = decltype(jt)::value;
+				if constexpr (j >= 2 && j < 10) ew_piece(1, j - 2);
+			};
+#pragma unroll
+			for (int f = 0; f < PA; ++f) read_a(0, f);
+			phase(na, [&](int f) __attribute__((always_inline)) { read_a(0, f); }, [&](int f) __attribute__((always_inline)) { prod_a(0, f); },
+			      [&](int f) __attribute__((always_inline)) { read_a(1, f); }, v0);
+			phase(na, [&](int f) __attribute__((always_inline)) { read_a(1, f); }, [&](int f) __attribute__((always_inline)) { prod_a(1, f); },
+			      [&](int f) __attribute__((always_inline)) { read_c(0, f); }, v1);
+			phase(nc, [&](int f) __attribute__((always_inline)) { read_c(0, f); }, [&](int f) __attribute__((always_inline)) { prod_c(0, f); },
+			      [&](int f) __attribute__((always_inline)) { read_c(1, f); }, v2);
+			phase(nc, [&](int f) __attribute__((always_inline)) { read_c(1, f); }, [&](int f) __attribute__((always_inline)) { prod_c(1, f); },
+			      [&](int) __attribute__((always_inline)) {}, none);
+			__builtin_amdgcn_sched_barrier(0);
+		}
+	};
+
 	// One pipeline step: publish tile t, start the copies of tile t + 1, compute.
 	auto step = [&](auto masked_tag, int t) {
 		const int n0 = t * BN;
@@ -1166,7 +1298,12 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 		}
 		bool skip = false;
 		if constexpr (decltype(masked_tag)::value) skip = n0 > wave_jmax || n0 + BN - 1 < wave_lmin;  // whole tile masked for this wave (uniform)
-		if (!skip) tile_body(masked_tag, n0);
+		if (!skip) {
+			if constexpr (PIPE && !decltype(masked_tag)::value)
+				tile_pipe(n0);
+			else
+				tile_body(masked_tag, n0);
+		}
 		// the other buffers next time
 #pragma unroll
 		for (int ks = 0; ks < KR; ++ks) koff[ks] ^= TILE_BYTES;
