@@ -78,6 +78,11 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	// dS = P * (dP accumulator).  The factor c1 = scale * log2(e) is applied to the fp32
 	// accumulator, as the reference scales the fp32 result of its dot (_backward_triton.py:554-559).
 	constexpr bool FOLD = KV_AGPR;
+	// Head dim 256: dK / dV fill the accumulation registers, and for S / dP - results that the vector ALU consumes - this
+	// compiler still chooses accumulation registers: it moves 32 registers of dK / dV out of the way and back in every
+	// block and copies S / dP out value by value (96 extra vector-ALU instructions per block of 16 values).  Their products
+	// are therefore issued as inline assembly with the accumulator pinned to a vector register.
+	constexpr bool S_VGPR = !KV_AGPR && D == 256 && !BIAS;  // (with a bias as well the pinned form runs out of vector registers)
 
 	// A bias in the element type of q is streamed through LDS as tiles of BMQ rows x BN keys
 	// where LDS has the room (the launcher then guarantees 16-byte aligned rows and whole key
@@ -421,6 +426,15 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 					mfma32_va<true>(dpa, afr[r], vf[ks]);
 				else
 					mfma32_va<true>(sa, afr[r], kf[ks]);
+			} else if constexpr (S_VGPR) {
+				if (j == 0)
+					mfma32_vz(sa, afr[r], kf[ks]);
+				else if (j == 1)
+					mfma32_vz(dpa, afr[r], vf[ks]);
+				else if (j & 1)
+					mfma32_va<false>(dpa, afr[r], vf[ks]);
+				else
+					mfma32_va<false>(sa, afr[r], kf[ks]);
 			} else {
 				// too many registers to pin: leave the register files to the compiler
 				f32x16 zero;
@@ -595,6 +609,9 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 			constexpr bool HAS_A = k < QB, HAS_B = k >= 1 && k - 1 < QB, HAS_C = k >= 2 && k - 2 < QB;
 			constexpr bool NEXT_A = k + 1 < QB, NEXT_B = k + 1 >= 1 && k < QB, NEXT_C = k + 1 >= 2 && k - 1 < QB;
 			__builtin_amdgcn_sched_barrier(0);
+			// (a stage that starts with the elementwise math of a block whose last products - inline assembly - were the
+			// previous stage's last instructions: their results need their wait states)
+			if constexpr (S_VGPR && HAS_B && !HAS_A) asm volatile("s_nop 15" ::: "memory");
 #pragma unroll
 			for (int j = 0; j < NSLOT; ++j) {
 				// LDS reads for the slot PA places ahead (in this stage or the next one)

@@ -71,6 +71,7 @@ FA2_DEV f32x16 mfma32(f16x8 a, f16x8 b, f32x16 c) {
 // least two further matrix products away from the product that wrote it.
 //   mfma32_va: C(VGPR) += A(VGPR) * B(AGPR)
 //   mfma32_vc: C(VGPR) = A(VGPR) * B(AGPR) + C0(VGPR)   first product of a chain, from a start value
+//   mfma32_vz: C(VGPR) = A(VGPR) * B(VGPR)              first product of a chain, from zero
 //   mfma32_aa: C(AGPR) += A(VGPR) * B(VGPR)
 // BA: the B operand lives in an AGPR (else in a VGPR)
 template <bool BA>
@@ -87,6 +88,9 @@ FA2_DEV void mfma32_va(f32x16& c, f16x8 a, f16x8 b) {
 	else
 		asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
 }
+// first product of a chain that starts from zero: C(VGPR) = A(VGPR) * B(VGPR)
+FA2_DEV void mfma32_vz(f32x16& c, bf16x8 a, bf16x8 b) { asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b)); }
+FA2_DEV void mfma32_vz(f32x16& c, f16x8 a, f16x8 b) { asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b)); }
 FA2_DEV void mfma32_vc(f32x16& c, bf16x8 a, bf16x8 b, f32x16 c0) {
 	asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(c) : "v"(a), "a"(b), "v"(c0));
 }
