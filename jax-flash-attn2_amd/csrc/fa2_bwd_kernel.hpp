@@ -82,7 +82,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	// compiler still chooses accumulation registers: it moves 32 registers of dK / dV out of the way and back in every
 	// block and copies S / dP out value by value (96 extra vector-ALU instructions per block of 16 values).  Their products
 	// are therefore issued as inline assembly with the accumulator pinned to a vector register.
-	constexpr bool S_VGPR = !KV_AGPR && D == 256 && !BIAS;  // (with a bias as well the pinned form runs out of vector registers)
+	constexpr bool S_VGPR = !KV_AGPR && ((D == 256 && !BIAS) || (D == 128 && BIAS && !DROP));  // (the other variants run out of vector registers in the pinned form)
 
 	// A bias in the element type of q is streamed through LDS as tiles of BMQ rows x BN keys
 	// where LDS has the room (the launcher then guarantees 16-byte aligned rows and whole key
