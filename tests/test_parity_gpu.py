@@ -60,6 +60,9 @@ def test_large_logits(dtype, qk_scale, score_range):
 	_run_case(1, 200, 333, 4, 4, 64, dtype, causal=False, qk_scale=qk_scale, data_seed=1)
 	_run_case(1, 160, 160, 2, 1, 256, dtype, causal=True, qk_scale=qk_scale, data_seed=2)
 	_run_case(1, 160, 160, 2, 2, 128, dtype, causal=True, qk_scale=qk_scale, p=0.1, seed=5, data_seed=3)
+	# head dim 256, many tiles without masking: the row reference has to be raised in later tiles too (with and without dropout)
+	_run_case(1, 96, 448, 2, 1, 256, dtype, causal=False, qk_scale=qk_scale, p=0.1, seed=7, data_seed=4)
+	_run_case(1, 72, 520, 2, 2, 256, dtype, causal=False, qk_scale=qk_scale, data_seed=5)
 
 
 @pytest.mark.parametrize(
@@ -316,6 +319,7 @@ def test_sliding_window(window):
 		(1, 192, 192, 2, 2, 256, torch.bfloat16, False, None, 0.0),
 		(2, 160, 224, 4, 2, 64, torch.bfloat16, False, (2, 1), 0.0),
 		(1, 192, 192, 4, 2, 128, torch.bfloat16, False, None, 0.2),
+		(1, 320, 448, 2, 1, 256, torch.bfloat16, False, None, 0.1),
 	)
 	for (B, Sq, Sk, Hq, Hkv, D, dtype, causal, bh, p) in cases:
 		bias_shape = None if bh is None else (*bh, Sq, Sk)
