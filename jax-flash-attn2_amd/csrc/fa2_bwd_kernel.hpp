@@ -608,28 +608,42 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 			constexpr int k = decltype(k_tag)::value;
 			constexpr bool HAS_A = k < QB, HAS_B = k >= 1 && k - 1 < QB, HAS_C = k >= 2 && k - 2 < QB;
 			constexpr bool NEXT_A = k + 1 < QB, NEXT_B = k + 1 >= 1 && k < QB, NEXT_C = k + 1 >= 2 && k - 1 < QB;
+			// One row block per step (head dim 256): nothing else is in flight, so the products of C start half a stage
+			// early - those of the block's first 16 rows (its slots 0 .. H - 1) run beside the elementwise math of its last
+			// 16 rows in the second half of stage 1, the rest in a stage 2 of half the length.
+			constexpr bool HALF = QB == 1;
+			constexpr int H = NSLOT / 2;
+			constexpr int NS = (HALF && k == 2) ? H : NSLOT;
 			__builtin_amdgcn_sched_barrier(0);
 			// (a stage that starts with the elementwise math of a block whose last products - inline assembly - were the
 			// previous stage's last instructions: their results need their wait states)
 			if constexpr (S_VGPR && HAS_B && !HAS_A) asm volatile("s_nop 15" ::: "memory");
 #pragma unroll
-			for (int j = 0; j < NSLOT; ++j) {
+			for (int j = 0; j < NS; ++j) {
+				// this slot's product of C, if any: block and slot index within that block's C
+				const bool has_c = HALF ? ((k == 1 && j >= H) || k == 2) : HAS_C;
+				const int cblk = HALF ? 0 : k - 2, jc = HALF ? (k == 1 ? j - H : j + H) : j;
 				// LDS reads for the slot PA places ahead (in this stage or the next one)
 				{
 					int jn = j + PA;
 					if (jn < NSLOT) {
 						if constexpr (HAS_A) issue_A(k, jn);
-						if constexpr (HAS_C) issue_C(k - 2, jn);
+						if constexpr (HAS_C && !HALF) issue_C(k - 2, jn);
 						if constexpr (HAS_B && !FOLD) {
 							issue_stat_for_slot(k - 1, jn);
 						}
 					} else {
 						int jj = jn - NSLOT;
 						if constexpr (NEXT_A) issue_A(k + 1, jj);
-						if constexpr (NEXT_C) issue_C(k - 1, jj);
+						if constexpr (NEXT_C && !HALF) issue_C(k - 1, jj);
 						if constexpr (NEXT_B && !FOLD) {
 							issue_stat_for_slot(k, jj);
 						}
+					}
+					if constexpr (HALF && k >= 1) {
+						// (stage 1 slot t is slot t - H of C, stage 2 slot t is slot t + H)
+						int cn = k == 1 ? j + PA - H : j + PA + H;
+						if (cn >= 0 && cn < NSLOT) issue_C(0, cn);
 					}
 					// the start values of the chains of the next block, in the last four slots
 					if constexpr (FOLD && NEXT_A) {
@@ -675,7 +689,9 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 				if constexpr (HAS_A && HAS_B) __builtin_amdgcn_sched_barrier(0);
 				b_half(0, 2);
 				if constexpr (HAS_A && HAS_C) __builtin_amdgcn_sched_barrier(0);
-				if constexpr (HAS_C) mfma_C(k - 2, j, pbits[k & 1], sbits[k & 1]);
+				if constexpr (HAS_C || (HALF && k >= 1)) {
+					if (has_c) mfma_C(cblk, jc, pbits[HALF ? 0 : (k & 1)], sbits[HALF ? 0 : (k & 1)]);
+				}
 				b_half(2, 4);
 				if constexpr (HAS_B && DROP) {
 					if constexpr (NSLOT >= 16) {
