@@ -78,10 +78,11 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	// dS = P * (dP accumulator).  The factor c1 = scale * log2(e) is applied to the fp32
 	// accumulator, as the reference scales the fp32 result of its dot (_backward_triton.py:554-559).
 	constexpr bool FOLD = KV_AGPR;
-	// Head dim 256: dK / dV fill the accumulation registers, and for S / dP - results that the vector ALU consumes - this
-	// compiler still chooses accumulation registers: it moves 32 registers of dK / dV out of the way and back in every
-	// block and copies S / dP out value by value (96 extra vector-ALU instructions per block of 16 values).  Their products
-	// are therefore issued as inline assembly with the accumulator pinned to a vector register.
+	// Where the register files are left to the compiler it chooses accumulation registers for S / dP as well - results
+	// that the vector ALU consumes - and copies them out value by value; at head dim 256, where dK / dV fill the
+	// accumulation registers, it also moves 32 registers of dK / dV out of the way and back in every block (96 extra
+	// vector-ALU instructions per block of 16 values).  For the variants named here the products of S / dP are therefore
+	// issued as inline assembly with the accumulator pinned to vector registers.
 	constexpr bool S_VGPR = !KV_AGPR && ((D == 256 && !BIAS) || (D == 128 && BIAS && !DROP));  // (the other variants run out of vector registers in the pinned form)
 
 	// A bias in the element type of q is streamed through LDS as tiles of BMQ rows x BN keys

@@ -403,7 +403,7 @@ FA2_DEV uint32_t quad_swap1(uint32_t x) { return (uint32_t)__builtin_amdgcn_mov_
 // the row's four values for keys jb + 8 aa .. + 3.  SHARE: the lane of the even row evaluates the calls of aa = 0, 2,
 // the lane of the odd row those of aa = 1, 3, and they exchange (needs lane ^ 1 = row ^ 1 in the same (b, h));
 // otherwise every lane evaluates its four calls itself.
-// One half of that: the words of aa = 2 pr and 2 pr + 1 (with SHARE one generator call per lane).
+// This function yields one half of that - w[0], w[1] = the words of aa = 2 pr and 2 pr + 1 (with SHARE one generator call per lane).
 template <bool SHARE>
 FA2_DEV void dropout_words_rowlane_half(int jb, uint32_t row, uint32_t h, uint32_t b, uint32_t k0, uint32_t k1, int pr, uint32_t (&w)[2][2]) {
 	const bool odd = row & 1u;
@@ -425,6 +425,7 @@ FA2_DEV void dropout_words_rowlane_half(int jb, uint32_t row, uint32_t h, uint32
 		}
 	}
 }
+// both halves: w[aa] for aa = 0 .. 3
 template <bool SHARE>
 FA2_DEV void dropout_words_rowlane(int jb, uint32_t row, uint32_t h, uint32_t b, uint32_t k0, uint32_t k1, uint32_t (&w)[4][2]) {
 #pragma unroll
