@@ -241,13 +241,15 @@ def attention_fwd(q, k, v, bias=None, causal=False, scale=None, seqlens=None,
 
 def attention_bwd(q, k, v, dO, bias=None, causal=False, scale=None, seqlens=None,
                   p_drop=0.0, seed=0, dtype=np.float64, pos_offset=(0, 0, 0), kv_lens=None, window=None, softcap=0.0,
-                  return_dbias=False):
+                  return_dbias=False, o_stored=None):
 	"""Analytic gradients (dQ, dK, dV) of sum(O * dO); FlashAttention-2 Algorithm 2,
 	the same five products as flash_attention_jax/_backward_jax.py:111-127, with
 	dK/dV summed over the q-heads of each KV group (_backward_triton.py:1156-1161).
 	No gradient for mask / seed (_flash_attention.py:88, _backward_jax.py:164).  The reference returns none for the
 	bias either; `return_dbias` adds it as a fourth result: dS = P (dP - delta) before the scale, summed over the
-	axes the bias is broadcast on (a size-1 batch or head axis, the q-heads of a KV group for a bias with Hkv heads)."""
+	axes the bias is broadcast on (a size-1 batch or head axis, the q-heads of a KV group for a bias with Hkv heads).
+	`o_stored`: the forward output as the backward pass receives it from the residuals (_flash_attention.py:68-75:
+	the stored O, rounded to its element type), used for delta = rowsum(O * dO); default: the exact O."""
 	B, Sq, Hq, D = q.shape
 	Sk, Hkv = k.shape[1], k.shape[2]
 	scale = (1.0 / math.sqrt(D)) if scale is None else scale
@@ -264,6 +266,8 @@ def attention_bwd(q, k, v, dO, bias=None, causal=False, scale=None, seqlens=None
 		dp = np.where(keep, dpd, 0.0) / dtype(1.0 - float(np.float32(p_drop)))
 	else:
 		dp = dpd
+	if o_stored is not None:
+		o = np.asarray(o_stored, dtype=dtype)
 	delta = np.einsum("bihd,bihd->bhi", o, dOf)[..., None]  # = rowsum(P * dP)
 	ds = p * (dp - delta)
 	dbias = None

@@ -44,15 +44,18 @@ def check_forward(o, lse, o_ref, lse_ref, dtype, what=""):
 		assert e <= TOL_LSE, f"{what}: LSE max-abs {e:.3e}"
 
 
-def check_grads(got, ref, what=""):
-	for name, a, b in zip(("dq", "dk", "dv"), got, ref):
+def check_grads(got, ref, what="", stored=None):
+	"""stored: the oracle's gradients with delta formed from O as the backward pass really receives it (rounded to
+	16 bits) - the size of what legitimately survives where the exact gradient cancels to zero."""
+	for n, (name, a, b) in enumerate(zip(("dq", "dk", "dv"), got, ref)):
 		a = a.float().cpu().numpy()
 		assert np.isfinite(a).all(), f"{what}: non-finite {name}"
 		if np.abs(b).max() <= 1e-10:
 			# a gradient that is zero up to fp64 rounding (e.g. a single key: dS = P (dP - delta) = 0) may come
 			# back as rounding noise of delta
-			# (delta is formed from O rounded to 16 bits: up to 2^-8 of |dP| survives the subtraction)
-			assert np.abs(a).max() <= 1e-2, f"{what}: {name} should be zero"
+			# (delta is formed from O rounded to 16 bits: up to 2^-8 of |dP| survives the subtraction, summed over the rows)
+			floor = 0.0 if stored is None else float(np.abs(stored[n]).max())
+			assert np.abs(a).max() <= 1e-2 + 2.0 * floor, f"{what}: {name} should be zero (max-abs {np.abs(a).max():.3e}, rounding floor {floor:.3e})"
 			continue
 		e = O.rel_l2(a, b)
 		assert e <= TOL_GRAD_REL_L2, f"{what}: {name} rel-L2 {e:.3e} > {TOL_GRAD_REL_L2}"

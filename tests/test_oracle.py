@@ -336,3 +336,24 @@ def test_golden_fixtures(name):
 		B, Sq, Hq, _ = z["q"].shape
 		keep = O.dropout_keep_mask(int(z["seed"]), float(z["p_drop"]), B, Hq, Sq, z["k"].shape[1])
 		assert np.array_equal(np.unpackbits(z["keep_bits"])[: keep.size].astype(bool).reshape(keep.shape), keep)
+
+
+def test_backward_with_the_stored_output():
+	"""`o_stored` only replaces O in delta = rowsum(O * dO): the exact O reproduces the default result, and with a single
+	key (P = 1) the exact gradients of q and k cancel to zero while a rounded O leaves its rounding error, summed over the rows."""
+	rng = np.random.default_rng(5)
+	q, k, v, do = (rng.standard_normal(s) for s in ((2, 9, 2, 8), (2, 5, 1, 8), (2, 5, 1, 8), (2, 9, 2, 8)))
+	o, _ = O.attention_fwd(q, k, v, causal=True)
+	ref = O.attention_bwd(q, k, v, do, causal=True)
+	same = O.attention_bwd(q, k, v, do, causal=True, o_stored=o)
+	for a, b in zip(ref, same):
+		assert np.array_equal(a, b)
+	k1, v1 = k[:, :1], v[:, :1]
+	o1, _ = O.attention_fwd(q, k1, v1)
+	exact = O.attention_bwd(q, k1, v1, do)
+	assert np.abs(exact[0]).max() <= 1e-12 and np.abs(exact[1]).max() <= 1e-12
+	noisy = O.attention_bwd(q, k1, v1, do, o_stored=o1 + 1e-3)
+	delta_err = 1e-3 * do.sum(-1)  # [B, Sq, H]: the error of delta; dS = -P * that, P = 1
+	want_dq = -delta_err[..., None] * np.repeat(k1, 2, axis=2) / np.sqrt(8)
+	assert np.allclose(noisy[0], want_dq, atol=1e-12)
+	assert np.allclose(noisy[2], exact[2])  # dV does not involve delta
