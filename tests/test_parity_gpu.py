@@ -179,6 +179,57 @@ def test_random_configurations(chunk):
 		_run_case(**_random_case(rng))
 
 
+def _run_extra_case(rng):
+	"""One configuration drawn from the operands that `_random_case` leaves out: key lengths, sliding window,
+	soft-capping (with and without a bias) and the bias gradient, in any combination with causal, dropout, GQA."""
+	r = int(rng.choice([1, 2, 4]))
+	Hkv = int(rng.choice([1, 2]))
+	Hq = Hkv * r
+	B = int(rng.choice([1, 2, 3]))
+	D = int(rng.choice([64, 128, 256]))
+	dtype = torch.bfloat16 if rng.random() < 0.6 else torch.float16
+	Sq = int(rng.integers(1, 330))
+	Sk = Sq if rng.random() < 0.5 else int(rng.integers(1, 700))
+	causal = bool(rng.random() < 0.4)
+	p = float(rng.choice([0.0, 0.0, 0.15]))
+	window = None
+	if rng.random() < 0.5:
+		window = (int(rng.choice([-1, 0, 7, 64, 150, 400])), int(rng.choice([-1, 0, 3, 64, 200])))
+	softcap = float(rng.choice([0.0, 0.0, 2.0, 20.0]))
+	with_bias = (softcap > 0 and rng.random() < 0.5) or rng.random() < 0.3
+	bias_shape = (int(rng.choice([1, B])), int(rng.choice([1, Hq])), Sq, Sk) if with_bias else None
+	kv_lens = [int(rng.integers(0, Sk + 1)) for _ in range(B)] if rng.random() < 0.4 else None
+	need_dbias = bias_shape is not None and rng.random() < 0.5
+	seed = int(rng.integers(0, 2**31))
+	q, k, v, do, bias = make_inputs(B, Sq, Sk, Hq, Hkv, D, dtype, int(rng.integers(0, 1000)), bias_shape)
+	kw = dict(causal=causal, p_drop=p, seed=seed, kv_lens=kv_lens, window=window, softcap=softcap)
+	what = (f"B{B} Sq{Sq} Sk{Sk} Hq{Hq} Hkv{Hkv} D{D} {dtype} causal={causal} p={p} window={window} softcap={softcap} "
+	        f"bias={bias_shape} kv_lens={kv_lens} dbias={need_dbias}")
+	o_ref, lse_ref = O.attention_fwd(f64(q), f64(k), f64(v), f64(bias), **kw)
+	g_ref = O.attention_bwd(f64(q), f64(k), f64(v), f64(do), f64(bias), return_dbias=need_dbias, **kw)
+	kl = None if kv_lens is None else torch.tensor(kv_lens, dtype=torch.int32, device=DEV)
+	o, lse = op.fwd(_dev(q), _dev(k), _dev(v), _dev(bias), None, None, p, causal, seed, kl, window, softcap)
+	g = op.bwd(_dev(q), _dev(k), _dev(v), o, lse, _dev(do), _dev(bias), None, None, p, causal, seed, kl, window, softcap, need_dbias)
+	torch.cuda.synchronize()
+	check_forward(o, lse, o_ref, lse_ref, dtype, what)
+	stored = None
+	if min(np.abs(x).max() for x in g_ref[:3]) <= 1e-10:
+		o_st = torch.from_numpy(np.nan_to_num(o_ref)).to(dtype).to(torch.float64).numpy()
+		stored = O.attention_bwd(f64(q), f64(k), f64(v), f64(do), f64(bias), o_stored=o_st, **kw)
+	check_grads(g[:3], g_ref[:3], what, stored)
+	if need_dbias and np.abs(g_ref[3]).max() > 1e-10:
+		e = O.rel_l2(g[3].float().cpu().numpy(), g_ref[3])
+		assert e <= 1e-2, f"{what}: dbias rel-L2 {e:.3e}"
+
+
+@pytest.mark.parametrize("chunk", range(5))
+def test_random_configurations_of_the_further_operands(chunk):
+	"""Seeded sweep over key lengths, sliding windows, soft-capping and the bias gradient, combined at random."""
+	rng = np.random.default_rng(4000 + chunk)
+	for _ in range(8):
+		_run_extra_case(rng)
+
+
 @pytest.mark.parametrize("D", [32, 80, 96, 160, 192])
 def test_other_head_dims(D):
 	"""Head dims between the built ones are zero-padded by the host layer (the reference pads
