@@ -26,6 +26,7 @@ constexpr float kRescaleSlack = 8.f;
 // without bias: largest partial row sum of one tile of P = exp2(c1 S - c1 m) taken without looking at
 // the row maximum (fp16 holds values up to 65504)
 constexpr float kFastSum = 16384.f;
+constexpr int kNumCU = 256;  // compute units of the MI355X (tile-size choice for small grids)
 
 // blockIdx.x -> (row tile, q-head, batch).  With xcd_remap the workgroups of
 // one (batch, kv-head) - which share K and V - are kept on one XCD (hardware
@@ -1042,34 +1043,47 @@ hipError_t launch_fwd_split_t(bool bias, bool drop, KArgs& a, hipStream_t s) {
 	return hipGetLastError();
 }
 
-template <typename T, int D>
-hipError_t launch_fwd_t(bool bias, bool drop, KArgs& a, hipStream_t s) {
-	if (a.nsplit > 1) return launch_fwd_split_t<T, D>(bias, drop, a, s);
-	typedef FwdCfg<T, D> C;
-	a.mtiles = (a.Sq + C::BM - 1) / C::BM;
+// One tile configuration: NW waves x 32 rows per workgroup (WPS: launch bound, waves per SIMD).
+template <typename T, int D, int NW, int WPS>
+hipError_t launch_fwd_cfg(bool bias, bool drop, KArgs& a, hipStream_t s) {
+	constexpr int QB = 1, BM = NW * QB * 32;
+	a.mtiles = (a.Sq + BM - 1) / BM;
 	int groups = a.B * a.Hkv;
 	a.xcd_remap = (groups % 8 == 0) ? 1 : 0;
 	a.interleave = a.xcd_remap ? launch_order(a, a.Hq / a.Hkv, groups / 8, (int64_t)a.Sk * D * 4) : 1;
 	if (bias && a.bias_sh == 0 && a.B % 8 == 0) a.xcd_remap = a.kv_lens ? 3 : 2;
-	dim3 grid((unsigned)(a.mtiles * a.B * a.Hq)), block(C::NW * 64);
+	dim3 grid((unsigned)(a.mtiles * a.B * a.Hq)), block(NW * 64);
 	const bool blds = bias && a.bias_lds && D <= 128;
 	if (a.softcap > 0.f && drop)
-		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, C::WPS, true, true, false, false, true>), grid, block, 0, s, a);
+		hipLaunchKernelGGL((fwd_kernel<T, D, NW, QB, WPS, true, true, false, false, true>), grid, block, 0, s, a);
 	else if (a.softcap > 0.f)
-		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, C::WPS, true, false, false, false, true>), grid, block, 0, s, a);
+		hipLaunchKernelGGL((fwd_kernel<T, D, NW, QB, WPS, true, false, false, false, true>), grid, block, 0, s, a);
 	else if (blds && drop)
-		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, C::WPS, true, true, false, true>), grid, block, 0, s, a);
+		hipLaunchKernelGGL((fwd_kernel<T, D, NW, QB, WPS, true, true, false, true>), grid, block, 0, s, a);
 	else if (blds)
-		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, C::WPS, true, false, false, true>), grid, block, 0, s, a);
+		hipLaunchKernelGGL((fwd_kernel<T, D, NW, QB, WPS, true, false, false, true>), grid, block, 0, s, a);
 	else if (bias && drop)
-		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, C::WPS, true, true>), grid, block, 0, s, a);
+		hipLaunchKernelGGL((fwd_kernel<T, D, NW, QB, WPS, true, true>), grid, block, 0, s, a);
 	else if (bias)
-		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, C::WPS, true, false>), grid, block, 0, s, a);
+		hipLaunchKernelGGL((fwd_kernel<T, D, NW, QB, WPS, true, false>), grid, block, 0, s, a);
 	else if (drop)
-		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, C::WPS, false, true>), grid, block, 0, s, a);
+		hipLaunchKernelGGL((fwd_kernel<T, D, NW, QB, WPS, false, true>), grid, block, 0, s, a);
 	else
-		hipLaunchKernelGGL((fwd_kernel<T, D, C::NW, C::QB, C::WPS, false, false>), grid, block, 0, s, a);
+		hipLaunchKernelGGL((fwd_kernel<T, D, NW, QB, WPS, false, false>), grid, block, 0, s, a);
 	return hipGetLastError();
+}
+
+template <typename T, int D>
+hipError_t launch_fwd_t(bool bias, bool drop, KArgs& a, hipStream_t s) {
+	if (a.nsplit > 1) return launch_fwd_split_t<T, D>(bias, drop, a, s);
+	typedef FwdCfg<T, D> C;
+	if constexpr (C::NW == 8) {
+		// A grid that leaves at least half of the chip idle (small batch x heads, short sequences): workgroups of
+		// 128 rows instead of 256, twice as many of them, still at most one per CU.
+		int64_t wgs = (int64_t)((a.Sq + 127) / 128) * a.B * a.Hq;
+		if (wgs <= kNumCU) return launch_fwd_cfg<T, D, 4, 1>(bias, drop, a, s);
+	}
+	return launch_fwd_cfg<T, D, C::NW, C::WPS>(bias, drop, a, s);
 }
 
 }  // namespace fa2
