@@ -1409,20 +1409,29 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 		constexpr int RPB = 256 / (D / 8);
 		hipLaunchKernelGGL((bwd_delta_kernel<T, D>), dim3((unsigned)((nrows + RPB - 1) / RPB)), dim3(256), 0, s, a);
 	}
-	auto launch_dq = [&]() {
-		a.mtiles = (a.Sq + C::DQ_BM - 1) / C::DQ_BM;
+	auto launch_dq_cfg = [&](auto nw_tag) {
+		constexpr int NW = decltype(nw_tag)::value, BM = NW * C::DQ_QB * 32;
+		a.mtiles = (a.Sq + BM - 1) / BM;
 		a.interleave = a.xcd_remap == 1 ? launch_order(a, a.Hq / a.Hkv, groups / 8, (int64_t)a.Sk * D * 4) : 1;
-		dim3 grid((unsigned)(a.mtiles * a.B * a.Hq)), block(C::DQ_NW * 64);
+		dim3 grid((unsigned)(a.mtiles * a.B * a.Hq)), block(NW * 64);
 		if (BIAS && a.dbias && a.softcap > 0.f)
-			hipLaunchKernelGGL((bwd_dq_kernel<T, D, C::DQ_NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, false, BIAS, BIAS>), grid, block, 0, s, a);
+			hipLaunchKernelGGL((bwd_dq_kernel<T, D, NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, false, BIAS, BIAS>), grid, block, 0, s, a);
 		else if (BIAS && a.dbias)
-			hipLaunchKernelGGL((bwd_dq_kernel<T, D, C::DQ_NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, false, false, BIAS>), grid, block, 0, s, a);
+			hipLaunchKernelGGL((bwd_dq_kernel<T, D, NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, false, false, BIAS>), grid, block, 0, s, a);
 		else if (BIAS && a.softcap > 0.f)
-			hipLaunchKernelGGL((bwd_dq_kernel<T, D, C::DQ_NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, false, BIAS>), grid, block, 0, s, a);
+			hipLaunchKernelGGL((bwd_dq_kernel<T, D, NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, false, BIAS>), grid, block, 0, s, a);
 		else if (BIAS && a.bias_lds && D <= 128)
-			hipLaunchKernelGGL((bwd_dq_kernel<T, D, C::DQ_NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, BIAS>), grid, block, 0, s, a);
+			hipLaunchKernelGGL((bwd_dq_kernel<T, D, NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, BIAS>), grid, block, 0, s, a);
 		else
-			hipLaunchKernelGGL((bwd_dq_kernel<T, D, C::DQ_NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, false>), grid, block, 0, s, a);
+			hipLaunchKernelGGL((bwd_dq_kernel<T, D, NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, false>), grid, block, 0, s, a);
+	};
+	auto launch_dq = [&]() {
+		if constexpr (C::DQ_NW == 8) {
+			// a grid that leaves at least half of the chip idle: workgroups of 128 rows instead of 256 (see the forward)
+			int64_t wgs = (int64_t)((a.Sq + 127) / 128) * a.B * a.Hq;
+			if (wgs <= kNumCU) return launch_dq_cfg(std::integral_constant<int, 4>{});
+		}
+		launch_dq_cfg(std::integral_constant<int, C::DQ_NW>{});
 	};
 	if (fused_delta) launch_dq();
 	if (a.stages & 2) {
