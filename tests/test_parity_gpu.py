@@ -222,6 +222,37 @@ def _run_extra_case(rng):
 		assert e <= 1e-2, f"{what}: dbias rel-L2 {e:.3e}"
 
 
+@pytest.mark.parametrize("D,dtype", [(64, torch.bfloat16), (128, torch.bfloat16), (128, torch.float16), (64, torch.float16)])
+def test_grids_that_fill_the_chip(D, dtype):
+	"""The forward and dQ kernels tile the rows in 128 when that still gives at most one workgroup per CU, which is what
+	the small shapes of the other tests get; these shapes (B x Hq x ceil(Sq / 128) > 256) take the 256-row workgroups
+	with every kind of operand: causal, dropout, bias through LDS and loaded directly (fp32), key lengths, lengths,
+	sliding window, soft-capping with the bias gradient."""
+	B, Hq, Hkv, S = 4, 16, 4, 520
+	assert B * Hq * ((S + 127) // 128) > 256
+	_run_case(B, S, S, Hq, Hkv, D, dtype, causal=True)
+	_run_case(B, S, S, Hq, Hkv, D, dtype, causal=True, p=0.2, seed=3, data_seed=1)
+	_run_case(B, S, 456, Hq, Hkv, D, dtype, causal=False, bias_shape=(B, 1, S, 456), data_seed=2)
+	_run_case(B, S, 457, Hq, Hkv, D, dtype, causal=False, bias_shape=(1, Hq, S, 457), bias_dtype=torch.float32, p=0.1, seed=4, data_seed=3)
+	_run_case(B, S, S, Hq, Hkv, D, dtype, causal=True, seqlens=[520, 1, 300, 77], data_seed=4)
+	rng = np.random.default_rng(7)
+	for window, softcap, with_bias, kv_lens, need_dbias in (((150, 0), 0.0, False, None, False), ((-1, 64), 0.0, False, [520, 0, 333, 64], False),
+	                                                        (None, 5.0, True, None, True), ((64, 64), 20.0, False, [100, 520, 519, 3], False)):
+		bias_shape = (B, Hq, S, S) if with_bias else None
+		q, k, v, do, bias = make_inputs(B, S, S, Hq, Hkv, D, dtype, int(rng.integers(0, 1000)), bias_shape)
+		kw = dict(causal=False, p_drop=0.0, seed=0, kv_lens=kv_lens, window=window, softcap=softcap)
+		what = f"D{D} {dtype} window={window} softcap={softcap} bias={bias_shape} kv_lens={kv_lens} dbias={need_dbias}"
+		o_ref, lse_ref = O.attention_fwd(f64(q), f64(k), f64(v), f64(bias), **kw)
+		g_ref = O.attention_bwd(f64(q), f64(k), f64(v), f64(do), f64(bias), return_dbias=need_dbias, **kw)
+		kl = None if kv_lens is None else torch.tensor(kv_lens, dtype=torch.int32, device=DEV)
+		o, lse = op.fwd(_dev(q), _dev(k), _dev(v), _dev(bias), None, None, 0.0, False, 0, kl, window, softcap)
+		g = op.bwd(_dev(q), _dev(k), _dev(v), o, lse, _dev(do), _dev(bias), None, None, 0.0, False, 0, kl, window, softcap, need_dbias)
+		check_forward(o, lse, o_ref, lse_ref, dtype, what)
+		check_grads(g[:3], g_ref[:3], what)
+		if need_dbias:
+			assert O.rel_l2(g[3].float().cpu().numpy(), g_ref[3]) <= 1e-2, f"{what}: dbias"
+
+
 @pytest.mark.parametrize("chunk", range(5))
 def test_random_configurations_of_the_further_operands(chunk):
 	"""Seeded sweep over key lengths, sliding windows, soft-capping and the bias gradient, combined at random."""
