@@ -201,6 +201,29 @@ size_t fa2_bwd_scratch_bytes(const fa2_params* p) {
 	return (n + 255) & ~(size_t)255;
 }
 
+// dK/dV on a small grid: B * Hkv * ceil(Sk / 128) workgroups that leave at least half of the chip idle, with several
+// q-heads per kv-head - the q-heads of a group are then split over 2, 4 .. workgroups (a power of two dividing the
+// group size) whose fp32 partial dK / dV a reduce kernel sums.  Returns the number of parts (1 = no split).
+static int bwd_head_split(const fa2_params* p) {
+	if (p->Hkv <= 0 || p->Hq % p->Hkv) return 1;
+	int r = p->Hq / p->Hkv;
+	long wgs = (long)p->B * p->Hkv * ((p->Sk + 127) / 128);
+	int hs = 1;
+	while (r % (hs * 2) == 0 && wgs * hs * 2 <= 256) hs *= 2;
+	return hs;
+}
+
+static size_t bwd_split_part_bytes(const fa2_params* p, int hs) {
+	return (size_t)hs * (size_t)p->B * (size_t)p->Hkv * (size_t)p->Sk * 2 * (size_t)p->D * sizeof(float);
+}
+
+size_t fa2_bwd_split_scratch_bytes(const fa2_params* p) {
+	size_t base = fa2_bwd_scratch_bytes(p);
+	if (!base || p->Sk <= 0 || p->D <= 0) return 0;
+	int hs = bwd_head_split(p);
+	return hs > 1 ? base + bwd_split_part_bytes(p, hs) : 0;
+}
+
 // Key ranges for a split forward: few query rows (one row tile of 64), too few (batch, head)
 // pairs to fill the chip, many keys.  Returns the number of ranges (1 = no split).
 // the rows of all q-heads of a kv-head fit one row tile: they share one workgroup (and one pass over K, V)
@@ -255,10 +278,21 @@ int fa2_fwd(const fa2_params* p, void* hip_stream) {
 
 int fa2_bwd(const fa2_params* p, void* hip_stream) { return fa2_bwd_stages(p, hip_stream, 7); }
 
-static int bwd_launch(const fa2_params* p, void* hip_stream, int stages, void* scratch_ptr) {
+static int bwd_launch(const fa2_params* p, void* hip_stream, int stages, void* scratch_ptr, size_t scratch_bytes) {
 	KArgs a;
 	fill(p, a);
 	a.stages = stages & 7;
+	// optional: with enough scratch behind delta the dK/dV kernel of a small grid runs split over the q-heads of a group
+	a.kv_hsplit = 1;
+	a.dkv_part = nullptr;
+	{
+		int hs = bwd_head_split(p);
+		size_t base = fa2_bwd_scratch_bytes(p);
+		if (hs > 1 && scratch_bytes >= base + bwd_split_part_bytes(p, hs)) {
+			a.kv_hsplit = hs;
+			a.dkv_part = (float*)((char*)scratch_ptr + base);
+		}
+	}
 	a.dout = conv(p->dout);
 	a.dq = conv(p->dq);
 	a.dk = conv(p->dk);
@@ -277,7 +311,7 @@ int fa2_bwd_stages(const fa2_params* p, void* hip_stream, int stages) {
 	p = complete(p, lp);
 	int rc = validate(p, 1);
 	if (rc) return rc;
-	return bwd_launch(p, hip_stream, stages, p->scratch);
+	return bwd_launch(p, hip_stream, stages, p->scratch, (size_t)p->scratch_bytes);
 }
 
 // Device address of `scratch` on the current device, looked up once per device.
@@ -305,7 +339,7 @@ int fa2_bwd_static(const fa2_params* p, void* hip_stream) {
 	void* ptr = nullptr;
 	if ((rc = static_scratch_ptr(&ptr))) return rc;
 	// delta is written in full by the first kernel before the second reads it: nothing to clear
-	return bwd_launch(p, hip_stream, 7, ptr);
+	return bwd_launch(p, hip_stream, 7, ptr, (size_t)FA2_STATIC_SCRATCH_BYTES);
 }
 
 int fa2_dropout_mask(const fa2_params* p, uint8_t* keep, void* hip_stream) {

@@ -106,7 +106,6 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	// "nothing to do for this wave") then stays in scalar registers and scalar branches
 	const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int g = lane >> 5, c = lane & 31;
-	const int r = a.Hq / a.Hkv;
 	// dropout key: from the parameter block, or from device memory when the caller keeps it there
 	uint32_t drop_k0 = a.drop_k0, drop_k1 = a.drop_k1;
 	if constexpr (DROP) {
@@ -117,9 +116,12 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	}
 
 	// blockIdx.x -> (key tile, kv head, batch); key tiles of one (b, kv head) stay on one XCD
+	// (with the q-heads of a group split over workgroups: the parts of one key tile are adjacent)
 	int nt, hk, b;
+	const int hsplit = a.kv_hsplit > 1 ? a.kv_hsplit : 1;
+	const int hsi = hsplit > 1 ? (int)blockIdx.x % hsplit : 0;
 	{
-		int id = blockIdx.x;
+		int id = hsplit > 1 ? (int)blockIdx.x / hsplit : (int)blockIdx.x;
 		int per_group = a.mtiles;
 		int grp, within;
 		if (a.xcd_remap >= 2) {
@@ -150,6 +152,9 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		b = grp / a.Hkv;
 		nt = within;  // early key tiles see the most query rows under a causal mask: first
 	}
+	// this workgroup's q-heads: r of them, from h_first
+	const int r = (a.Hq / a.Hkv) / hsplit;
+	const int h_first = hk * (a.Hq / a.Hkv) + hsi * r;
 
 	int sq_eff = a.Sq, sk_eff = a.Sk;
 	if (a.seqlens) {
@@ -240,7 +245,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	// moment wait on each other.)
 	auto decode_step = [&](int step, int& hq, int& m0) __attribute__((always_inline)) {
 		int hi = step / nq;
-		hq = hk * r + hi;
+		hq = h_first + hi;
 		m0 = (q_lo + (step - hi * nq)) * BMQ;
 	};
 	// start the copies of streamed tile `step` (rows beyond Sq are fetched from the last valid row)
@@ -810,6 +815,21 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	// the last matrix products (issued as inline assembly) must have written dk / dv
 	asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 	// epilogue: lane owns key jcol, four consecutive d per store
+	if (hsplit > 1) {
+		// partial sums over this workgroup's q-heads, fp32 and unscaled, for the reduce kernel
+		if (jcol < a.Sk) {
+			float* pp = a.dkv_part + ((((int64_t)hsi * a.B + b) * a.Hkv + hk) * a.Sk + jcol) * (2 * D);
+#pragma unroll
+			for (int db = 0; db < DB; ++db)
+#pragma unroll
+				for (int aa = 0; aa < 4; ++aa) {
+					int d0 = 32 * db + 8 * aa + 4 * g;
+					*(f32x4*)(pp + d0) = f32x4{dk[db][4 * aa], dk[db][4 * aa + 1], dk[db][4 * aa + 2], dk[db][4 * aa + 3]};
+					*(f32x4*)(pp + D + d0) = f32x4{dv[db][4 * aa], dv[db][4 * aa + 1], dv[db][4 * aa + 2], dv[db][4 * aa + 3]};
+				}
+		}
+		return;
+	}
 	if (jcol < a.Sk) {
 		char* dkp = a.dk.ptr + (int64_t)b * a.dk.sb + (int64_t)hk * a.dk.sh + (int64_t)jcol * a.dk.ss;
 		char* dvp = a.dv.ptr + (int64_t)b * a.dv.sb + (int64_t)hk * a.dv.sh + (int64_t)jcol * a.dv.ss;
@@ -828,6 +848,41 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 				*(u32x2*)(dvp + d0 * 2) = pv;
 			}
 	}
+}
+
+// Sum of the partial dK / dV that a head-split dK/dV launch left (a.dkv_part, see KArgs), scaled and stored in the
+// element type: one thread per (batch, kv-head, key, dK | dV, eight consecutive d).
+template <typename T, int D>
+__global__ __launch_bounds__(256) void bwd_dkdv_reduce_kernel(const KArgs a, float dk_scale, float dv_scale) {
+	constexpr int CH = D / 8;  // chunks of eight per row
+	int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+	int64_t total = (int64_t)a.B * a.Hkv * a.Sk * 2 * CH;
+	if (idx >= total) return;
+	int ch = (int)(idx % CH);
+	int which = (int)((idx / CH) % 2);
+	int64_t row = idx / (2 * CH);  // (b * Hkv + hk) * Sk + key
+	int key = (int)(row % a.Sk);
+	int hk = (int)((row / a.Sk) % a.Hkv);
+	int b = (int)(row / ((int64_t)a.Sk * a.Hkv));
+	const int64_t part_stride = (int64_t)a.B * a.Hkv * a.Sk * 2 * D;
+	const float* pp = a.dkv_part + row * (2 * D) + which * D + ch * 8;
+	float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+	for (int s = 0; s < a.kv_hsplit; ++s) {
+		f32x4 x0 = *(const f32x4*)(pp + s * part_stride), x1 = *(const f32x4*)(pp + s * part_stride + 4);
+#pragma unroll
+		for (int e = 0; e < 4; ++e) {
+			acc[e] += x0[e];
+			acc[4 + e] += x1[e];
+		}
+	}
+	const float sc = which ? dv_scale : dk_scale;
+	const KTensor& out = which ? a.dv : a.dk;
+	u32x4 pk = {pack2<typename T::V2>(acc[0] * sc, acc[1] * sc), pack2<typename T::V2>(acc[2] * sc, acc[3] * sc),
+	            pack2<typename T::V2>(acc[4] * sc, acc[5] * sc), pack2<typename T::V2>(acc[6] * sc, acc[7] * sc)};
+	char* op_ = out.ptr + (int64_t)b * out.sb + (int64_t)hk * out.sh + (int64_t)key * out.ss + ch * 16;
+	// (rows of dk / dv need not be 16-byte aligned: two 8-byte stores)
+	*(u32x2*)op_ = u32x2{pk[0], pk[1]};
+	*(u32x2*)(op_ + 8) = u32x2{pk[2], pk[3]};
 }
 
 // ---------------------------------------------------------------------------
@@ -1437,7 +1492,8 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 	if (a.stages & 2) {
 		a.mtiles = (a.Sk + C::KV_BN - 1) / C::KV_BN;
 		a.interleave = a.xcd_remap == 1 ? launch_order(a, 1, groups / 8, (int64_t)(a.Hq / a.Hkv) * a.Sq * D * 4) : 1;
-		dim3 grid((unsigned)(a.mtiles * a.B * a.Hkv)), block(C::KV_NW * 64);
+		const int hs = a.kv_hsplit > 1 ? a.kv_hsplit : 1;
+		dim3 grid((unsigned)(a.mtiles * a.B * a.Hkv * hs)), block(C::KV_NW * 64);
 		// typed variant: bias in the element type of q; where it stages the bias through LDS (D <= 128)
 		// it also needs 16-byte aligned rows of whole 16-byte pieces
 		bool typed = BIAS && a.bias_dtype == (std::is_same<T, BF16>::value ? 2 : 1);
@@ -1450,6 +1506,11 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 			hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, C::KV_NW, QBV, BIAS, DROP, BIAS>), grid, block, 0, s, a);
 		else
 			hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, C::KV_NW, QBV, BIAS, DROP, false>), grid, block, 0, s, a);
+		if (hs > 1) {
+			int64_t total = (int64_t)a.B * a.Hkv * a.Sk * 2 * (D / 8);
+			hipLaunchKernelGGL((bwd_dkdv_reduce_kernel<T, D>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, a, a.scale,
+			                   DROP ? a.drop_inv_keep : 1.f);
+		}
 	}
 	if ((a.stages & 4) && !fused_delta) launch_dq();
 	return hipGetLastError();

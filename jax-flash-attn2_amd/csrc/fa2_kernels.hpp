@@ -40,6 +40,10 @@ struct KArgs {
 	int mtiles;      // number of row tiles of the launched kernel
 	int xcd_remap;   // 1: group-major placement of workgroups on the 8 XCDs
 	                 // 2: batch-major placement, heads of a row tile adjacent (a bias shared by the heads stays in L2)
+	// dK/dV kernel on small grids: the q-heads of a KV group are split over kv_hsplit workgroups, each leaving fp32
+	// partial dK / dV in dkv_part [kv_hsplit][B][Hkv][Sk][2][D]; a reduce kernel sums, scales and stores them.  1 = no split.
+	int kv_hsplit;
+	float* dkv_part;
 	int interleave;  // xcd_remap 1: this many (batch, kv-head) groups of an XCD advance through their tiles together (1, 2 or 4)
 	int stages;      // backward: bit 0 delta, bit 1 dK/dV, bit 2 dQ
 	int dq_makes_delta;  // the dQ kernel computes delta itself (and stores it for the dK/dV kernel)

@@ -191,7 +191,8 @@ def bwd(q, k, v, out, lse, dout, bias=None, seqlens=None, softmax_scale=None, dr
 	p.o = _t4(out)
 	p.lse = lse.data_ptr()
 	p.dout, p.dq, p.dk, p.dv = _t4(dout), _t4(dq), _t4(dk), _t4(dv)
-	need = lib.fa2_bwd_scratch_bytes(ctypes.byref(p))
+	# (the larger size, where it applies, lets the dK/dV kernel of a small grid split the q-heads of a group over workgroups)
+	need = max(lib.fa2_bwd_scratch_bytes(ctypes.byref(p)), lib.fa2_bwd_split_scratch_bytes(ctypes.byref(p)))
 	scratch = torch.empty((max(need, 256),), dtype=torch.uint8, device=q.device)
 	p.scratch = scratch.data_ptr()
 	p.scratch_bytes = scratch.numel()
@@ -267,7 +268,7 @@ class Plan:
 			self.dk = torch.empty_like(self.k, memory_format=torch.contiguous_format)
 			self.dv = torch.empty_like(self.v, memory_format=torch.contiguous_format)
 			p.dout, p.dq, p.dk, p.dv = _t4(self.dout), _t4(self.dq), _t4(self.dk), _t4(self.dv)
-			need = self.lib.fa2_bwd_scratch_bytes(ctypes.byref(p))
+			need = max(self.lib.fa2_bwd_scratch_bytes(ctypes.byref(p)), self.lib.fa2_bwd_split_scratch_bytes(ctypes.byref(p)))
 		else:
 			need = 0
 		# one buffer serves both calls: the backward needs its scratch, the forward uses scratch when it splits a

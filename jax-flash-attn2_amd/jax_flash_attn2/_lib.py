@@ -76,6 +76,7 @@ EXPORTS = (
 	"fa2_bwd_stages",
 	"fa2_bwd_static",
 	"fa2_bwd_scratch_bytes",
+	"fa2_bwd_split_scratch_bytes",
 	"fa2_fwd_scratch_bytes",
 	"fa2_dropout_mask",
 	"fa2_validate",
@@ -119,6 +120,8 @@ def load() -> ctypes.CDLL:
 		lib.fa2_bwd_static.restype = ctypes.c_int
 		lib.fa2_bwd_scratch_bytes.argtypes = [pp]
 		lib.fa2_bwd_scratch_bytes.restype = ctypes.c_size_t
+		lib.fa2_bwd_split_scratch_bytes.argtypes = [pp]
+		lib.fa2_bwd_split_scratch_bytes.restype = ctypes.c_size_t
 		lib.fa2_fwd_scratch_bytes.argtypes = [pp]
 		lib.fa2_fwd_scratch_bytes.restype = ctypes.c_size_t
 		lib.fa2_dropout_mask.argtypes = [pp, ctypes.c_void_p, ctypes.c_void_p]

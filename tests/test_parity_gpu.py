@@ -705,6 +705,41 @@ def test_backward_is_deterministic_and_outputs_fully_written():
 	assert torch.equal(plan.dq, a[0]) and torch.equal(plan.dk, a[1]) and torch.equal(plan.dv, a[2])
 
 
+@pytest.mark.parametrize("D,dtype,p_drop", [(128, torch.bfloat16, 0.0), (64, torch.float16, 0.1), (256, torch.bfloat16, 0.0)])
+def test_backward_with_and_without_the_head_split(D, dtype, p_drop):
+	"""On a small grid the dK/dV kernel splits the q-heads of a KV group over workgroups when the caller's scratch has
+	room for the partial sums (fa2_bwd_split_scratch_bytes), and runs unsplit with the minimum scratch: both give the
+	oracle's gradients, each bit-identical from call to call, and the partial buffer of a larger earlier call does not
+	leak into a smaller one."""
+	import ctypes
+	from jax_flash_attn2 import _lib
+	lib = _lib.load()
+	B, S, Hq, Hkv = 2, 333, 8, 2
+	q, k, v, do, _ = make_inputs(B, S, S, Hq, Hkv, D, dtype, 21)
+	kw = dict(causal=True, p_drop=p_drop, seed=6)
+	g_ref = O.attention_bwd(f64(q), f64(k), f64(v), f64(do), None, **kw)
+	plan = op.Plan(_dev(q), _dev(k), _dev(v), dout=_dev(do), causal=True, dropout_prob=p_drop, dropout_seed=6 if p_drop else None)
+	P = ctypes.byref(plan.params)
+	need_min, need_split = lib.fa2_bwd_scratch_bytes(P), lib.fa2_bwd_split_scratch_bytes(P)
+	assert need_split > need_min and plan.params.scratch_bytes >= need_split
+	plan.forward()
+	results = {}
+	for name, nbytes in (("split", plan.params.scratch_bytes), ("unsplit", need_min)):
+		plan.params.scratch_bytes = nbytes
+		runs = []
+		for _ in range(2):
+			for t in (plan.dq, plan.dk, plan.dv):
+				t.fill_(float("nan"))
+			plan.backward()
+			torch.cuda.synchronize()
+			runs.append([t.clone() for t in (plan.dq, plan.dk, plan.dv)])
+		for x, y in zip(*runs):
+			assert torch.equal(x, y), name
+		check_grads(runs[0], g_ref, f"{name} D{D} {dtype} p={p_drop}")
+		results[name] = runs[0]
+	assert torch.equal(results["split"][0], results["unsplit"][0])  # dQ does not depend on the split
+
+
 @pytest.mark.parametrize("order", [(1, 2, 4), (1, 4, 2), (5, 2), (3, 4), (1, 6)])
 def test_backward_by_stages_matches_the_oracle(order):
 	"""fa2_bwd_stages: the stand-alone delta pre-pass (bit 0), the dK/dV kernel (bit 1) and the dQ kernel (bit 2)
