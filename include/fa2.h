@@ -185,12 +185,12 @@ int fa2_bwd_stages(const fa2_params* p, void* hip_stream, int stages);
 size_t fa2_bwd_scratch_bytes(const fa2_params* p);
 
 /* Optional larger scratch for fa2_bwd / fa2_bwd_stages.  Non-zero when the dK/dV kernel's grid
- * (B * Hkv * ceil(Sk / 128) workgroups) would leave at least half of the chip idle and a KV
- * group has several q-heads: given `scratch` of at least this many bytes (it includes
- * fa2_bwd_scratch_bytes), the q-heads of a group are split over 2, 4 .. workgroups that leave
- * fp32 partial dK / dV behind delta, and a third kernel sums them in a fixed order (results
- * stay deterministic).  With less scratch the backward runs unsplit.  The reference has no
- * counterpart: it sums dK / dV over the q-heads on the host side of its launcher
+ * (B * Hkv * ceil(Sk / 128) workgroups) would leave at least half of the chip idle: given
+ * `scratch` of at least this many bytes (it includes fa2_bwd_scratch_bytes), the work of a key
+ * tile - the q-heads of its KV group times the query tiles - is split over up to 8 workgroups
+ * that leave fp32 partial dK / dV behind delta, and a third kernel sums them in a fixed order
+ * (results stay deterministic).  With less scratch the backward runs unsplit.  The reference
+ * has no counterpart: it sums dK / dV over the q-heads on the host side of its launcher
  * (_backward_triton.py:1156-1161).  0 when no split applies. */
 size_t fa2_bwd_split_scratch_bytes(const fa2_params* p);
 

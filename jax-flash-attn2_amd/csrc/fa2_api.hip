@@ -201,16 +201,17 @@ size_t fa2_bwd_scratch_bytes(const fa2_params* p) {
 	return (n + 255) & ~(size_t)255;
 }
 
-// dK/dV on a small grid: B * Hkv * ceil(Sk / 128) workgroups that leave at least half of the chip idle, with several
-// q-heads per kv-head - the q-heads of a group are then split over 2, 4 .. workgroups (a power of two dividing the
-// group size) whose fp32 partial dK / dV a reduce kernel sums.  Returns the number of parts (1 = no split).
-static int bwd_head_split(const fa2_params* p) {
+// dK/dV on a small grid: B * Hkv * ceil(Sk / 128) workgroups that leave at least half of the chip idle - the steps a
+// key tile streams (the q-heads of its KV group x the query tiles) are then split over up to 8 workgroups whose fp32
+// partial dK / dV a reduce kernel sums.  Returns the number of parts (1 = no split).
+static int bwd_step_split(const fa2_params* p) {
 	if (p->Hkv <= 0 || p->Hq % p->Hkv) return 1;
-	int r = p->Hq / p->Hkv;
 	long wgs = (long)p->B * p->Hkv * ((p->Sk + 127) / 128);
-	int hs = 1;
-	while (r % (hs * 2) == 0 && wgs * hs * 2 <= 256) hs *= 2;
-	return hs;
+	long steps = (long)(p->Hq / p->Hkv) * ((p->Sq + 127) / 128);  // of the longest key tile, in units of 128 rows
+	long parts = wgs > 0 ? 256 / wgs : 1;
+	if (parts > 8) parts = 8;
+	if (parts > steps) parts = steps;
+	return parts >= 2 ? (int)parts : 1;
 }
 
 static size_t bwd_split_part_bytes(const fa2_params* p, int hs) {
@@ -220,7 +221,7 @@ static size_t bwd_split_part_bytes(const fa2_params* p, int hs) {
 size_t fa2_bwd_split_scratch_bytes(const fa2_params* p) {
 	size_t base = fa2_bwd_scratch_bytes(p);
 	if (!base || p->Sk <= 0 || p->D <= 0) return 0;
-	int hs = bwd_head_split(p);
+	int hs = bwd_step_split(p);
 	return hs > 1 ? base + bwd_split_part_bytes(p, hs) : 0;
 }
 
@@ -286,7 +287,7 @@ static int bwd_launch(const fa2_params* p, void* hip_stream, int stages, void* s
 	a.kv_hsplit = 1;
 	a.dkv_part = nullptr;
 	{
-		int hs = bwd_head_split(p);
+		int hs = bwd_step_split(p);
 		size_t base = fa2_bwd_scratch_bytes(p);
 		if (hs > 1 && scratch_bytes >= base + bwd_split_part_bytes(p, hs)) {
 			a.kv_hsplit = hs;

@@ -116,7 +116,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	}
 
 	// blockIdx.x -> (key tile, kv head, batch); key tiles of one (b, kv head) stay on one XCD
-	// (with the q-heads of a group split over workgroups: the parts of one key tile are adjacent)
+	// (with the steps of a key tile split over workgroups: the parts of one key tile are adjacent)
 	int nt, hk, b;
 	const int hsplit = a.kv_hsplit > 1 ? a.kv_hsplit : 1;
 	const int hsi = hsplit > 1 ? (int)blockIdx.x % hsplit : 0;
@@ -152,9 +152,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		b = grp / a.Hkv;
 		nt = within;  // early key tiles see the most query rows under a causal mask: first
 	}
-	// this workgroup's q-heads: r of them, from h_first
-	const int r = (a.Hq / a.Hkv) / hsplit;
-	const int h_first = hk * (a.Hq / a.Hkv) + hsi * r;
+	const int r = a.Hq / a.Hkv;
 
 	int sq_eff = a.Sq, sk_eff = a.Sk;
 	if (a.seqlens) {
@@ -228,6 +226,9 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	if (jcol >= sk_eff) row_lo = 1 << 30;
 	const int nq = q_hi > q_lo ? q_hi - q_lo : 0;
 	const int steps = nq * r;
+	// this workgroup's share of the steps (all of them unless the launch splits the steps of a key tile over `hsplit` workgroups)
+	const int s_lo = hsplit > 1 ? (int)((int64_t)steps * hsi / hsplit) : 0;
+	const int s_hi = hsplit > 1 ? (int)((int64_t)steps * (hsi + 1) / hsplit) : steps;
 
 	const float c1 = BIAS ? a.scale : a.scale * kLog2e;
 	const float inv_scale = 1.f / a.scale;
@@ -245,7 +246,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	// moment wait on each other.)
 	auto decode_step = [&](int step, int& hq, int& m0) __attribute__((always_inline)) {
 		int hi = step / nq;
-		hq = h_first + hi;
+		hq = hk * r + hi;
 		m0 = (q_lo + (step - hi * nq)) * BMQ;
 	};
 	// start the copies of streamed tile `step` (rows beyond Sq are fetched from the last valid row)
@@ -260,7 +261,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		if constexpr (BIAS_LDS) {
 			int hb = a.bias_group ? hk : hq;
 			const char* bb_ = a.bias + (int64_t)b * a.bias_sb + (int64_t)hb * a.bias_sh + (int64_t)m0 * a.bias_sm + (int64_t)n0 * 2;
-			bload.load(lds_bias + (step & 1) * BIAS_BYTES, bb_, a.bias_sm, rows, tid, (a.Sk - n0) >> 3);
+			bload.load(lds_bias + ((step - s_lo) & 1) * BIAS_BYTES, bb_, a.bias_sm, rows, tid, (a.Sk - n0) >> 3);
 		}
 	};
 	// per-row statistics of a tile: thread t < BMQ fetches lse, t in [BMQ, 2 BMQ) fetches delta.
@@ -735,18 +736,18 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		static_assert(QB <= 4, "");
 	};
 
-	if (steps > 0) {
-		issue_tile(0, lds, lds + TILE_BYTES);
-		store_stat(fetch_stat(0), 0);
+	if (s_hi > s_lo) {
+		issue_tile(s_lo, lds, lds + TILE_BYTES);
+		store_stat(fetch_stat(s_lo), 0);
 	}
 
 	// One pipeline step: publish streamed tile `step`, start the copies of the next, compute.
 	auto run_step = [&](auto masked_tag, int step) {
-		const int buf = step & 1;
+		const int buf = (step - s_lo) & 1;
 		wait_async_loads();
 		__syncthreads();
 		float next_stat = 0.f;
-		const bool has_next = step + 1 < steps;
+		const bool has_next = step + 1 < s_hi;
 		if (has_next) {
 			// statistics first: loads return in order, so waiting for this small load later
 			// does not wait for the tile copies issued after it
@@ -806,17 +807,19 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	i_diag = i_diag < 0 ? 0 : (i_diag > nq ? nq : i_diag);
 	i_full = i_full < i_diag ? i_diag : (i_full > nq ? nq : i_full);
 	for (int hi = 0; hi < r && nq > 0; ++hi) {
+		// (each of the three runs clipped to this workgroup's share of the steps)
 		int base = hi * nq;
-		for (int i = 0; i < i_diag; ++i) run_step(std::true_type{}, base + i);
-		for (int i = i_diag; i < i_full; ++i) run_step(std::false_type{}, base + i);
-		for (int i = i_full; i < nq; ++i) run_step(std::true_type{}, base + i);
+		auto clip = [&](int i) { int st = base + i; return st < s_lo ? s_lo : (st > s_hi ? s_hi : st); };
+		for (int st = clip(0); st < clip(i_diag); ++st) run_step(std::true_type{}, st);
+		for (int st = clip(i_diag); st < clip(i_full); ++st) run_step(std::false_type{}, st);
+		for (int st = clip(i_full); st < clip(nq); ++st) run_step(std::true_type{}, st);
 	}
 
 	// the last matrix products (issued as inline assembly) must have written dk / dv
 	asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 	// epilogue: lane owns key jcol, four consecutive d per store
 	if (hsplit > 1) {
-		// partial sums over this workgroup's q-heads, fp32 and unscaled, for the reduce kernel
+		// partial sums over this workgroup's share of the steps, fp32 and unscaled, for the reduce kernel
 		if (jcol < a.Sk) {
 			float* pp = a.dkv_part + ((((int64_t)hsi * a.B + b) * a.Hkv + hk) * a.Sk + jcol) * (2 * D);
 #pragma unroll
@@ -850,7 +853,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	}
 }
 
-// Sum of the partial dK / dV that a head-split dK/dV launch left (a.dkv_part, see KArgs), scaled and stored in the
+// Sum of the partial dK / dV that a dK/dV launch with split steps left (a.dkv_part, see KArgs), scaled and stored in the
 // element type: one thread per (batch, kv-head, key, dK | dV, eight consecutive d).
 template <typename T, int D>
 __global__ __launch_bounds__(256) void bwd_dkdv_reduce_kernel(const KArgs a, float dk_scale, float dv_scale) {

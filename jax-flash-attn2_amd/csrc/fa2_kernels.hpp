@@ -40,8 +40,9 @@ struct KArgs {
 	int mtiles;      // number of row tiles of the launched kernel
 	int xcd_remap;   // 1: group-major placement of workgroups on the 8 XCDs
 	                 // 2: batch-major placement, heads of a row tile adjacent (a bias shared by the heads stays in L2)
-	// dK/dV kernel on small grids: the q-heads of a KV group are split over kv_hsplit workgroups, each leaving fp32
-	// partial dK / dV in dkv_part [kv_hsplit][B][Hkv][Sk][2][D]; a reduce kernel sums, scales and stores them.  1 = no split.
+	// dK/dV kernel on small grids: the streamed steps of a key tile (q-heads of the KV group x query tiles) are split
+	// over kv_hsplit workgroups, each leaving fp32 partial dK / dV in dkv_part [kv_hsplit][B][Hkv][Sk][2][D]; a reduce
+	// kernel sums, scales and stores them.  1 = no split.
 	int kv_hsplit;
 	float* dkv_part;
 	int interleave;  // xcd_remap 1: this many (batch, kv-head) groups of an XCD advance through their tiles together (1, 2 or 4)

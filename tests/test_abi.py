@@ -190,9 +190,9 @@ def test_forward_scratch_only_for_short_queries_over_many_keys():
 	assert need(1, 65, 8192, 8) == 0             # more than one row tile of 64
 
 
-def test_backward_split_scratch_only_on_small_grids_with_grouped_heads():
-	"""fa2_bwd_split_scratch_bytes: non-zero exactly where the dK/dV kernel may split the q-heads of a group over
-	workgroups - delta plus one fp32 [B, Hkv, Sk, 2, D] partial per part."""
+def test_backward_split_scratch_only_on_small_grids():
+	"""fa2_bwd_split_scratch_bytes: non-zero exactly where the dK/dV kernel may split the steps of a key tile over
+	workgroups - delta plus one fp32 [B, Hkv, Sk, 2, D] partial per part (at most 8, at most 256 workgroups in all)."""
 	lib = _lib.load()
 
 	def need(B, S, Hq, Hkv, D=128):
@@ -201,10 +201,12 @@ def test_backward_split_scratch_only_on_small_grids_with_grouped_heads():
 		return lib.fa2_bwd_split_scratch_bytes(ctypes.byref(p)), lib.fa2_bwd_scratch_bytes(ctypes.byref(p))
 
 	assert need(4, 4096, 32, 8)[0] == 0        # 4 x 8 x 32 workgroups fill the chip
-	assert need(1, 2048, 8, 8)[0] == 0         # one q-head per kv-head: nothing to split
-	n, base = need(1, 2048, 16, 4)             # 1 x 4 x 16 = 64 workgroups, groups of 4: 4 parts
+	assert need(1, 4096, 32, 8)[0] == 0        # 256 workgroups: one per CU already
+	n, base = need(1, 2048, 16, 4)             # 1 x 4 x 16 = 64 workgroups: 4 parts
 	assert n == base + 4 * (1 * 4 * 2048 * 2 * 128 * 4)
-	n, base = need(1, 2048, 32, 8)             # 128 workgroups: 2 parts
+	n, base = need(1, 2048, 8, 8)              # 128 workgroups: 2 parts, also with one q-head per kv-head
 	assert n == base + 2 * (1 * 8 * 2048 * 2 * 128 * 4)
-	n, base = need(1, 512, 6, 2, 64)           # groups of 3: no power of two divides them
+	n, base = need(1, 512, 6, 2, 64)           # 8 workgroups: the limit of 8 parts
+	assert n == base + 8 * (1 * 2 * 512 * 2 * 64 * 4)
+	n, base = need(1, 100, 2, 2)               # a single step per key tile: nothing to split
 	assert n == 0

@@ -706,11 +706,10 @@ def test_backward_is_deterministic_and_outputs_fully_written():
 
 
 @pytest.mark.parametrize("D,dtype,p_drop", [(128, torch.bfloat16, 0.0), (64, torch.float16, 0.1), (256, torch.bfloat16, 0.0)])
-def test_backward_with_and_without_the_head_split(D, dtype, p_drop):
-	"""On a small grid the dK/dV kernel splits the q-heads of a KV group over workgroups when the caller's scratch has
-	room for the partial sums (fa2_bwd_split_scratch_bytes), and runs unsplit with the minimum scratch: both give the
-	oracle's gradients, each bit-identical from call to call, and the partial buffer of a larger earlier call does not
-	leak into a smaller one."""
+def test_backward_with_and_without_the_step_split(D, dtype, p_drop):
+	"""On a small grid the dK/dV kernel splits the steps of a key tile (q-heads of the group x query tiles) over
+	workgroups when the caller's scratch has room for the partial sums (fa2_bwd_split_scratch_bytes), and runs unsplit
+	with the minimum scratch: both give the oracle's gradients, each bit-identical from call to call."""
 	import ctypes
 	from jax_flash_attn2 import _lib
 	lib = _lib.load()
