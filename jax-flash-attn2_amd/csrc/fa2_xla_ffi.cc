@@ -20,7 +20,7 @@
 // (_forward_triton.py:553): a new seed then needs no new executable and the seed may be traced.
 // All tensors are dense row-major as XLA lays them out: q/o/dout/dq [B,Sq,Hq,D],
 // k/v/dk/dv [B,Sk,Hkv,D], bias [B|1, H|1, Sq, Sk], lse [B,Hq,Sq] f32,
-// scratch u8: fa2_bwd_scratch_bytes for the backward, fa2_fwd_scratch_bytes (or any smaller size: no split) for the forward.
+// scratch u8: fa2_bwd_scratch_bytes (or the larger fa2_bwd_split_scratch_bytes) for the backward, fa2_fwd_scratch_bytes (or any smaller size: no split) for the forward.
 #include <hip/hip_runtime.h>
 
 #include <cstring>

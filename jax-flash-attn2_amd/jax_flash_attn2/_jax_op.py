@@ -118,6 +118,20 @@ def _fwd_scratch_bytes(q, k) -> int:
 	return max(int(_lib.load().fa2_fwd_scratch_bytes(ctypes.byref(p))), 256)
 
 
+def _bwd_scratch_bytes(q, k) -> int:
+	"""Scratch of the backward for these shapes (host-only query): fa2_bwd_scratch_bytes, or the larger
+	fa2_bwd_split_scratch_bytes where the dK/dV kernel can split a key tile's work over workgroups."""
+	import ctypes
+
+	from . import _lib
+
+	p = _lib.new_params()
+	p.B, p.Sq, p.Hq, p.D = (int(x) for x in q.shape)
+	p.Sk, p.Hkv = int(k.shape[1]), int(k.shape[2])
+	lib = _lib.load()
+	return max(int(lib.fa2_bwd_scratch_bytes(ctypes.byref(p))), int(lib.fa2_bwd_split_scratch_bytes(ctypes.byref(p))), 256)
+
+
 def _fwd_call(q, k, v, bias, seqlens, seed, attrs):
 	_register()
 	B, Sq, Hq, _ = q.shape
@@ -132,8 +146,7 @@ def _fwd_call(q, k, v, bias, seqlens, seed, attrs):
 
 def _bwd_call(q, k, v, bias, seqlens, seed, out, lse, dout, attrs):
 	_register()
-	B, Sq, Hq, _ = q.shape
-	scratch_bytes = (B * Hq * Sq * 4 + 255) // 256 * 256  # fa2_bwd_scratch_bytes
+	scratch_bytes = _bwd_scratch_bytes(q, k)
 	out_types = (
 		jax.ShapeDtypeStruct(q.shape, q.dtype),
 		jax.ShapeDtypeStruct(k.shape, k.dtype),
