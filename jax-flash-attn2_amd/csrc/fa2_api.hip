@@ -210,7 +210,10 @@ static int bwd_step_split(const fa2_params* p) {
 	long steps = (long)(p->Hq / p->Hkv) * ((p->Sq + 127) / 128);  // of the longest key tile, in units of 128 rows
 	long parts = wgs > 0 ? 256 / wgs : 1;
 	if (parts > 8) parts = 8;
-	if (parts > steps) parts = steps;
+	// (the partial sums and their reduction have a fixed cost - about 5 us: measured, a key tile of fewer than 8 such steps
+	// is faster unsplit, and a part should have at least two)
+	if (steps < 8) return 1;
+	if (parts > steps / 2) parts = steps / 2;
 	return parts >= 2 ? (int)parts : 1;
 }
 
@@ -234,8 +237,8 @@ static bool fwd_pack_gqa(const fa2_params* p) {
 
 static int fwd_split_plan(const fa2_params* p, int* split_len) {
 	*split_len = 0;
-	if (p->Sq > 64) return 1;
-	long base = (long)p->B * (fwd_pack_gqa(p) ? p->Hkv : p->Hq);
+	// workgroups of an unsplit launch of this kernel variant (row tiles of 64)
+	long base = fwd_pack_gqa(p) ? (long)p->B * p->Hkv : (long)p->B * p->Hq * ((p->Sq + 63) / 64);
 	int tiles = (p->Sk + 63) / 64;
 	if (base >= 512 || tiles < 8) return 1;
 	long want = (1024 + base - 1) / base;

@@ -171,8 +171,8 @@ def test_missing_library_fails_loudly(monkeypatch):
 		_lib.load()
 
 
-def test_forward_scratch_only_for_short_queries_over_many_keys():
-	"""fa2_fwd_scratch_bytes: non-zero exactly where the split forward applies."""
+def test_forward_scratch_only_for_small_grids_over_many_keys():
+	"""fa2_fwd_scratch_bytes: non-zero exactly where the split forward applies (too few row tiles to fill the chip, many keys)."""
 	lib = _lib.load()
 
 	def need(B, Sq, Sk, Hq, D=128):
@@ -187,7 +187,9 @@ def test_forward_scratch_only_for_short_queries_over_many_keys():
 	assert n > 0 and n % 256 == 0
 	# ranges x rows x (D values + logsumexp) floats, rounded up to 256 bytes
 	assert n >= 2 * 8 * (128 + 1) * 4 and n <= 64 * 8 * (128 + 1) * 4 + 256
-	assert need(1, 65, 8192, 8) == 0             # more than one row tile of 64
+	n2 = need(1, 65, 8192, 8)                    # two row tiles of 64: still far from filling the chip
+	assert n2 > 0 and n2 % 256 == 0
+	assert need(1, 4096, 4096, 8) == 0           # 512 row tiles of 64: enough already
 
 
 def test_backward_split_scratch_only_on_small_grids():
@@ -206,7 +208,9 @@ def test_backward_split_scratch_only_on_small_grids():
 	assert n == base + 4 * (1 * 4 * 2048 * 2 * 128 * 4)
 	n, base = need(1, 2048, 8, 8)              # 128 workgroups: 2 parts, also with one q-head per kv-head
 	assert n == base + 2 * (1 * 8 * 2048 * 2 * 128 * 4)
-	n, base = need(1, 512, 6, 2, 64)           # 8 workgroups: the limit of 8 parts
-	assert n == base + 8 * (1 * 2 * 512 * 2 * 64 * 4)
-	n, base = need(1, 100, 2, 2)               # a single step per key tile: nothing to split
-	assert n == 0
+	n, base = need(1, 1024, 12, 2, 64)         # 16 workgroups: the limit of 8 parts
+	assert n == base + 8 * (1 * 2 * 1024 * 2 * 64 * 4)
+	n, base = need(1, 512, 6, 2, 64)           # 12 steps of 128 rows per key tile: at most 6 parts
+	assert n == base + 6 * (1 * 2 * 512 * 2 * 64 * 4)
+	assert need(2, 512, 8, 8)[0] == 0          # only 4 steps per key tile: the split would cost more than it saves
+	assert need(1, 100, 2, 2)[0] == 0
