@@ -158,9 +158,9 @@ typedef struct fa2_params {
  * Replaces the `_attn_fwd` custom call (_forward_triton.py:547-588). */
 int fa2_fwd(const fa2_params* p, void* hip_stream);
 
-/* Optional scratch for fa2_fwd.  Non-zero for many keys (>= 512) under too few (batch, head,
- * 64-row tile) units to fill the chip - decoding, `Sq == 1` in flash_attention.py:239-242,
- * and short prompts at batch 1 with few heads: given `scratch` (256-byte aligned) of at least this many
+/* Optional scratch for fa2_fwd.  Non-zero for many keys under too few (batch, head, 64-row tile)
+ * units to fill the chip - decoding, `Sq == 1` in flash_attention.py:239-242, from 512 keys, and
+ * prompts at batch 1 with few heads from 1024 or 2048 keys: given `scratch` (256-byte aligned) of at least this many
  * bytes, fa2_fwd splits the keys into ranges handled by separate workgroups and merges the
  * partial results (same O and lse to rounding).  Without it the call runs unsplit. */
 size_t fa2_fwd_scratch_bytes(const fa2_params* p);

@@ -240,7 +240,12 @@ static int fwd_split_plan(const fa2_params* p, int* split_len) {
 	// workgroups of an unsplit launch of this kernel variant (row tiles of 64)
 	long base = fwd_pack_gqa(p) ? (long)p->B * p->Hkv : (long)p->B * p->Hq * ((p->Sq + 63) / 64);
 	int tiles = (p->Sk + 63) / 64;
-	if (base >= 512 || tiles < 8) return 1;
+	// A query longer than one row tile runs unsplit on the 128-row kernel, which a quarter of the chip's worth of
+	// units already keeps busy over a short key range: the second launch pays from 16 key tiles on up to 128 units
+	// and from 32 above (measured at D=64: 256 units over 16 tiles 0.0185 ms unsplit, 0.0203 ms split; over 32 tiles
+	// 0.0316 and 0.0235).
+	int min_tiles = p->Sq <= 64 ? 8 : (base <= 128 ? 16 : 32);
+	if (base >= 512 || tiles < min_tiles) return 1;
 	long want = (1024 + base - 1) / base;
 	if (want > tiles / 4) want = tiles / 4;
 	if (want > 64) want = 64;

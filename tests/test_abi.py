@@ -190,6 +190,10 @@ def test_forward_scratch_only_for_small_grids_over_many_keys():
 	n2 = need(1, 65, 8192, 8)                    # two row tiles of 64: still far from filling the chip
 	assert n2 > 0 and n2 % 256 == 0
 	assert need(1, 4096, 4096, 8) == 0           # 512 row tiles of 64: enough already
+	assert need(2, 512, 512, 16, 64) == 0        # 256 row tiles over 8 key tiles: too short a kernel for a second launch
+	assert need(1, 1024, 1024, 16, 64) == 0      # 256 row tiles over 16 key tiles: the same
+	assert need(1, 2048, 2048, 8, 64) > 0        # 256 row tiles over 32 key tiles: split
+	assert need(1, 1024, 1024, 8, 64) > 0        # 128 row tiles over 16 key tiles: split
 
 
 def test_backward_split_scratch_only_on_small_grids():
