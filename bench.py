@@ -178,6 +178,30 @@ def cpu_baseline(w):
 	return out
 
 
+def reference_grid(torch, op, dev, args):
+	"""Forward-only times over the shapes named by the result files under the reference's benchmarks/
+	(`b=<B>-ub=<bias>-hdim=<D>-qh=<Hq>-kvh=<Hkv>-mode=fwd.csv`, rows seqlen 1024 ... 8192).  Those files record neither
+	dtype, causal flag nor the bias shape: here bf16, non-causal, bias [B, Hq, S, S] (the most traffic a bias can bring)."""
+	print("| B | bias | D | Hq | Hkv | S | ms | TFLOP/s |")
+	print("|---|---|---|---|---|---|---|---|")
+	for B in (1, 2, 4):
+		for ub in (False, True):
+			for D in (64, 128, 256):
+				for Hq, Hkv in ((16, 8), (32, 16)):
+					for S in (1024, 2048, 4096, 6144, 8192):
+						w = dict(B=B, S=S, Hq=Hq, Hkv=Hkv, D=D, dtype="bf16", causal=False, bias=False, p=0.0, bwd=False)
+						q, k, v, _, _, _ = make_inputs(w, dev)
+						bias = torch.empty((B, Hq, S, S), dtype=torch.bfloat16, device=dev).normal_() if ub else None
+						plan = op.Plan(q, k, v, bias=bias, causal=False)
+						t_pre = time.perf_counter()
+						while time.perf_counter() - t_pre < 0.1:
+							plan.forward()
+							torch.cuda.synchronize()
+						ms = event_time_ms(plan.forward, max(3, min(args.steps, 20)), torch)
+						print(f"| {B} | {'yes' if ub else 'no'} | {D} | {Hq} | {Hkv} | {S} | {ms:.4f} | {fwd_flops(w) / (ms * 1e-3) / 1e12:.0f} |", flush=True)
+						del plan, q, k, v, bias
+
+
 def main():
 	ap = argparse.ArgumentParser()
 	ap.add_argument("--gpus", type=int, default=1)
@@ -191,6 +215,9 @@ def main():
 	ap.add_argument("--copy-calibration", action="store_true",
 	                help="also run a plain 1 GiB device copy (known traffic) so that rocprofv3 FETCH_SIZE / WRITE_SIZE "
 	                     "readings of the attention kernels can be scaled")
+	ap.add_argument("--reference-grid", action="store_true",
+	                help="instead of one workload: forward times over the grid of shapes the reference's benchmarks/ folder "
+	                     "holds results for (batch, bias, head dim, heads, sequence length); prints a markdown table")
 	args = ap.parse_args()
 	if args.gpus != 1:
 		print("bench.py: this build measures ONE GPU; --gpus N with N > 1 is not supported "
@@ -205,6 +232,9 @@ def main():
 		print("bench.py: no GPU visible", file=sys.stderr)
 		sys.exit(1)
 	dev = torch.device("cuda:0")
+	if args.reference_grid:
+		reference_grid(torch, op, dev, args)
+		return
 	w = WORKLOADS[args.workload]
 	q, k, v, do, bias, kv_lens = make_inputs(w, dev)
 	plan = op.Plan(q, k, v, dout=do if w["bwd"] else None, bias=bias, causal=w["causal"], dropout_prob=w["p"],

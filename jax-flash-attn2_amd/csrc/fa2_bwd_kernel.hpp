@@ -88,8 +88,9 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	// A bias in the element type of q is streamed through LDS as tiles of BMQ rows x BN keys
 	// where LDS has the room (the launcher then guarantees 16-byte aligned rows and whole key
 	// tiles): fetched one key per lane from global memory, every value is a 2-byte load of its own.
-	// (D = 128: LDS has room only with 64-row tiles, which the launcher chooses for bias; D = 256: no registers to spare)
-	constexpr bool BIAS_LDS = BIAS && BIAS_T && 4 * TILE_BYTES + 4 * STAT_BYTES + 2 * BMQ * BN * 2 <= 160 * 1024 && D <= 128;
+	// (D = 128: LDS has room only with 64-row tiles, which the launcher chooses for bias.  D = 256, 32-row tiles: through
+	// LDS the dK/dV kernel of B2 H16 S4096 with a bias per head takes 1.37 ms, with a load per value 4.12 ms.)
+	constexpr bool BIAS_LDS = BIAS && BIAS_T && 4 * TILE_BYTES + 4 * STAT_BYTES + 2 * BMQ * BN * 2 <= 160 * 1024;
 	constexpr int BIAS_BYTES = BIAS_LDS ? BMQ * BN * 2 : 0;
 	static_assert(BN == 128, "bias tiles use the 128-element row geometry");
 	// Q[0] dO[0] Q[1] dO[1] | lse[0] lse[1] delta[0] delta[1] | bias[0] bias[1]
@@ -907,7 +908,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 	constexpr int TILE_BYTES = BN * D * 2;
 
 	// bias tiles through LDS as in the forward kernel
-	constexpr bool BIAS_LDS = BIAS && BLDS && D <= 128;
+	constexpr bool BIAS_LDS = BIAS && BLDS;
 	constexpr int BIAS_BYTES = BIAS_LDS ? BM * BN * 2 : 0;
 	static_assert(BN == 64, "bias tiles use the 64-element row geometry");
 	__shared__ __attribute__((aligned(1024))) char smem[4 * TILE_BYTES + 2 * BIAS_BYTES];
@@ -1478,7 +1479,7 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 			hipLaunchKernelGGL((bwd_dq_kernel<T, D, NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, false, false, BIAS>), grid, block, 0, s, a);
 		else if (BIAS && a.softcap > 0.f)
 			hipLaunchKernelGGL((bwd_dq_kernel<T, D, NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, false, BIAS>), grid, block, 0, s, a);
-		else if (BIAS && a.bias_lds && D <= 128)
+		else if (BIAS && a.bias_lds)
 			hipLaunchKernelGGL((bwd_dq_kernel<T, D, NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, BIAS>), grid, block, 0, s, a);
 		else
 			hipLaunchKernelGGL((bwd_dq_kernel<T, D, NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, false>), grid, block, 0, s, a);
@@ -1497,10 +1498,9 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 		a.interleave = a.xcd_remap == 1 ? launch_order(a, 1, groups / 8, (int64_t)(a.Hq / a.Hkv) * a.Sq * D * 4) : 1;
 		const int hs = a.kv_hsplit > 1 ? a.kv_hsplit : 1;
 		dim3 grid((unsigned)(a.mtiles * a.B * a.Hkv * hs)), block(C::KV_NW * 64);
-		// typed variant: bias in the element type of q; where it stages the bias through LDS (D <= 128)
-		// it also needs 16-byte aligned rows of whole 16-byte pieces
+		// typed variant: bias in the element type of q, staged through LDS: it also needs 16-byte aligned rows of whole 16-byte pieces
 		bool typed = BIAS && a.bias_dtype == (std::is_same<T, BF16>::value ? 2 : 1);
-		if (D <= 128 && !a.bias_lds) typed = false;
+		if (!a.bias_lds) typed = false;
 		// with bias at D = 128 the streamed tiles are 64 rows, which leaves LDS room for the bias tiles
 		constexpr int QBV = (BIAS && D == 128) ? 2 : C::KV_QB;
 		if (BIAS && a.softcap > 0.f)

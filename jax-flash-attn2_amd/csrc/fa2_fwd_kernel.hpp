@@ -157,7 +157,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 
 	// Bias tiles (BM rows x 64 keys, element type of q) go through LDS as well when there is
 	// room: read from global memory one row per lane, a wave's load touches 32 cache lines.
-	constexpr bool BIAS_LDS = BIAS && BLDS && D <= 128;
+	constexpr bool BIAS_LDS = BIAS && BLDS && (D <= 128 || !SPLIT);
 	constexpr int BIAS_BYTES = BIAS_LDS ? BM * BN * 2 : 0;
 	static_assert(BN == 64, "bias tiles use the 64-element row geometry");
 	__shared__ __attribute__((aligned(1024))) char smem[4 * TILE_BYTES + 2 * BIAS_BYTES];
@@ -1053,7 +1053,7 @@ hipError_t launch_fwd_cfg(bool bias, bool drop, KArgs& a, hipStream_t s) {
 	a.interleave = a.xcd_remap ? launch_order(a, a.Hq / a.Hkv, groups / 8, (int64_t)a.Sk * D * 4) : 1;
 	if (bias && a.bias_sh == 0 && a.B % 8 == 0) a.xcd_remap = a.kv_lens ? 3 : 2;
 	dim3 grid((unsigned)(a.mtiles * a.B * a.Hq)), block(NW * 64);
-	const bool blds = bias && a.bias_lds && D <= 128;
+	const bool blds = bias && a.bias_lds;
 	if (a.softcap > 0.f && drop)
 		hipLaunchKernelGGL((fwd_kernel<T, D, NW, QB, WPS, true, true, false, false, true>), grid, block, 0, s, a);
 	else if (a.softcap > 0.f)
