@@ -185,7 +185,8 @@ int fa2_bwd_stages(const fa2_params* p, void* hip_stream, int stages);
 size_t fa2_bwd_scratch_bytes(const fa2_params* p);
 
 /* Optional larger scratch for fa2_bwd / fa2_bwd_stages.  Non-zero when the dK/dV kernel's grid
- * (B * Hkv * ceil(Sk / 128) workgroups) would leave at least half of the chip idle: given
+ * (B * Hkv * ceil(Sk / 128) workgroups) would leave at least half of the chip idle, or - causal,
+ * fewer than 512 workgroups of long key tiles - would leave it waiting for the longest: given
  * `scratch` of at least this many bytes (it includes fa2_bwd_scratch_bytes), the work of a key
  * tile - the q-heads of its KV group times the query tiles - is split over up to 8 workgroups
  * that leave fp32 partial dK / dV behind delta, and a third kernel sums them in a fixed order

@@ -208,7 +208,15 @@ static int bwd_step_split(const fa2_params* p) {
 	if (p->Hkv <= 0 || p->Hq % p->Hkv) return 1;
 	long wgs = (long)p->B * p->Hkv * ((p->Sk + 127) / 128);
 	long steps = (long)(p->Hq / p->Hkv) * ((p->Sq + 127) / 128);  // of the longest key tile, in units of 128 rows
-	long parts = wgs > 0 ? 256 / wgs : 1;
+	long parts = wgs > 0 ? 256 / wgs : 1;  // fill the chip
+	if (p->causal && wgs < 512) {
+		// Causal key tiles differ in length (the first has all the steps, the last one row block's), and with at most
+		// two workgroups per CU the longest sets the time: about 1024 workgroups of at least 64 steps pack well
+		// (B4 Hq32 Hkv2 S4096 D128: dK/dV 1.56 ms unsplit, 1.06 ms in 4 parts; Hkv1 3.00 and 1.07 ms in 8 parts).
+		long bal = (1024 + wgs / 2) / wgs;
+		if (bal > steps / 64) bal = steps / 64;
+		if (bal > parts) parts = bal;
+	}
 	if (parts > 8) parts = 8;
 	// (the partial sums and their reduction have a fixed cost - about 5 us: measured, a key tile of fewer than 8 such steps
 	// is faster unsplit, and a part should have at least two)

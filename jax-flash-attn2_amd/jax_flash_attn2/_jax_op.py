@@ -118,7 +118,7 @@ def _fwd_scratch_bytes(q, k) -> int:
 	return max(int(_lib.load().fa2_fwd_scratch_bytes(ctypes.byref(p))), 256)
 
 
-def _bwd_scratch_bytes(q, k) -> int:
+def _bwd_scratch_bytes(q, k, causal=False) -> int:
 	"""Scratch of the backward for these shapes (host-only query): fa2_bwd_scratch_bytes, or the larger
 	fa2_bwd_split_scratch_bytes where the dK/dV kernel can split a key tile's work over workgroups."""
 	import ctypes
@@ -128,6 +128,7 @@ def _bwd_scratch_bytes(q, k) -> int:
 	p = _lib.new_params()
 	p.B, p.Sq, p.Hq, p.D = (int(x) for x in q.shape)
 	p.Sk, p.Hkv = int(k.shape[1]), int(k.shape[2])
+	p.causal = 1 if causal else 0  # (causal launches split further: their key tiles differ in length)
 	lib = _lib.load()
 	return max(int(lib.fa2_bwd_scratch_bytes(ctypes.byref(p))), int(lib.fa2_bwd_split_scratch_bytes(ctypes.byref(p))), 256)
 
@@ -146,7 +147,7 @@ def _fwd_call(q, k, v, bias, seqlens, seed, attrs):
 
 def _bwd_call(q, k, v, bias, seqlens, seed, out, lse, dout, attrs):
 	_register()
-	scratch_bytes = _bwd_scratch_bytes(q, k)
+	scratch_bytes = _bwd_scratch_bytes(q, k, attrs["causal"])
 	out_types = (
 		jax.ShapeDtypeStruct(q.shape, q.dtype),
 		jax.ShapeDtypeStruct(k.shape, k.dtype),

@@ -198,12 +198,13 @@ def test_forward_scratch_only_for_small_grids_over_many_keys():
 
 def test_backward_split_scratch_only_on_small_grids():
 	"""fa2_bwd_split_scratch_bytes: non-zero exactly where the dK/dV kernel may split the steps of a key tile over
-	workgroups - delta plus one fp32 [B, Hkv, Sk, 2, D] partial per part (at most 8, at most 256 workgroups in all)."""
+	workgroups - delta plus one fp32 [B, Hkv, Sk, 2, D] partial per part (at most 8; enough to fill the chip and, for causal
+	launches, to even out key tiles of different length)."""
 	lib = _lib.load()
 
-	def need(B, S, Hq, Hkv, D=128):
+	def need(B, S, Hq, Hkv, D=128, causal=0):
 		p = _lib.new_params()
-		p.B, p.Sq, p.Sk, p.Hq, p.Hkv, p.D = B, S, S, Hq, Hkv, D
+		p.B, p.Sq, p.Sk, p.Hq, p.Hkv, p.D, p.causal = B, S, S, Hq, Hkv, D, causal
 		return lib.fa2_bwd_split_scratch_bytes(ctypes.byref(p)), lib.fa2_bwd_scratch_bytes(ctypes.byref(p))
 
 	assert need(4, 4096, 32, 8)[0] == 0        # 4 x 8 x 32 workgroups fill the chip
@@ -218,3 +219,16 @@ def test_backward_split_scratch_only_on_small_grids():
 	assert n == base + 6 * (1 * 2 * 512 * 2 * 64 * 4)
 	assert need(2, 512, 8, 8)[0] == 0          # only 4 steps per key tile: the split would cost more than it saves
 	assert need(1, 100, 2, 2)[0] == 0
+	# causal key tiles differ in length: fewer than 512 workgroups are split further, towards 1024 parts of at least 64 steps
+	n, base = need(1, 4096, 32, 8, causal=1)   # 256 workgroups, 128 steps: 2 parts
+	assert n == base + 2 * (1 * 8 * 4096 * 2 * 128 * 4)
+	n, base = need(4, 4096, 32, 2, causal=1)   # 256 workgroups, 512 steps: 4 parts
+	assert n == base + 4 * (4 * 2 * 4096 * 2 * 128 * 4)
+	n, base = need(4, 4096, 32, 1, causal=1)   # 128 workgroups, 1024 steps: 8 parts
+	assert n == base + 8 * (4 * 1 * 4096 * 2 * 128 * 4)
+	n, base = need(3, 4096, 32, 4, causal=1)   # 384 workgroups: 3 parts
+	assert n == base + 3 * (3 * 4 * 4096 * 2 * 128 * 4)
+	assert need(2, 4096, 32, 8, causal=1)[0] == 0   # 512 workgroups pack well unsplit
+	assert need(4, 4096, 32, 8, causal=1)[0] == 0
+	n, base = need(1, 2048, 8, 8, causal=1)    # 16 steps: the 2 parts that fill the chip, no more
+	assert n == base + 2 * (1 * 8 * 2048 * 2 * 128 * 4)

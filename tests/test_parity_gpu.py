@@ -739,6 +739,41 @@ def test_backward_with_and_without_the_step_split(D, dtype, p_drop):
 	assert torch.equal(results["split"][0], results["unsplit"][0])  # dQ does not depend on the split
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,S,D,parts", [(1, 32, 8, 4096, 128, 2), (2, 16, 1, 4096, 64, 8), (3, 16, 4, 4096, 256, 2)])
+def test_step_split_of_a_causal_grid_near_the_cu_count(B, Hq, Hkv, S, D, parts):
+	"""Causal grids of fewer than 512 key-tile workgroups are split further than filling the chip needs (their key tiles
+	differ in length).  At these sizes the oracle is out of reach: the split launch must reproduce the unsplit one, which
+	sums the same fp32 products in another order - dQ bit for bit, dK / dV to rounding of the 16-bit results."""
+	import ctypes
+	from jax_flash_attn2 import _lib
+	lib = _lib.load()
+	dev = torch.device("cuda:0")
+	g = torch.Generator(device=dev)
+	g.manual_seed(5)
+	rnd = lambda *shape: (torch.randn(shape, generator=g, device=dev, dtype=torch.float32) * 0.5).to(torch.bfloat16)
+	q, k, v, do = rnd(B, S, Hq, D), rnd(B, S, Hkv, D), rnd(B, S, Hkv, D), rnd(B, S, Hq, D)
+	plan = op.Plan(q, k, v, dout=do, causal=True)
+	P = ctypes.byref(plan.params)
+	need_min, need_split = lib.fa2_bwd_scratch_bytes(P), lib.fa2_bwd_split_scratch_bytes(P)
+	if parts:
+		assert need_split == need_min + parts * B * Hkv * S * 2 * D * 4
+	assert need_split > need_min and plan.params.scratch_bytes >= need_split
+	plan.forward()
+	results = {}
+	for name, nbytes in (("split", plan.params.scratch_bytes), ("unsplit", need_min)):
+		plan.params.scratch_bytes = nbytes
+		for t in (plan.dq, plan.dk, plan.dv):
+			t.fill_(float("nan"))
+		plan.backward()
+		torch.cuda.synchronize()
+		results[name] = [t.clone() for t in (plan.dq, plan.dk, plan.dv)]
+	assert torch.equal(results["split"][0], results["unsplit"][0])
+	for x, y, what in zip(results["split"][1:], results["unsplit"][1:], ("dk", "dv")):
+		assert torch.isfinite(x.float()).all(), what
+		rel = float((x.float() - y.float()).norm() / y.float().norm())
+		assert rel < 2e-3, (what, rel)  # (one rounding step of bf16 is 2^-9 = 2e-3 of a value; most values agree exactly)
+
+
 @pytest.mark.parametrize("order", [(1, 2, 4), (1, 4, 2), (5, 2), (3, 4), (1, 6)])
 def test_backward_by_stages_matches_the_oracle(order):
 	"""fa2_bwd_stages: the stand-alone delta pre-pass (bit 0), the dK/dV kernel (bit 1) and the dQ kernel (bit 2)
