@@ -1468,29 +1468,36 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 		constexpr int RPB = 256 / (D / 8);
 		hipLaunchKernelGGL((bwd_delta_kernel<T, D>), dim3((unsigned)((nrows + RPB - 1) / RPB)), dim3(256), 0, s, a);
 	}
-	auto launch_dq_cfg = [&](auto nw_tag) {
-		constexpr int NW = decltype(nw_tag)::value, BM = NW * C::DQ_QB * 32;
+	auto launch_dq_cfg = [&](auto nw_tag, auto wps_tag) {
+		constexpr int NW = decltype(nw_tag)::value, BM = NW * C::DQ_QB * 32, WPS = decltype(wps_tag)::value;
 		a.mtiles = (a.Sq + BM - 1) / BM;
 		a.interleave = a.xcd_remap == 1 ? launch_order(a, a.Hq / a.Hkv, groups / 8, (int64_t)a.Sk * D * 4) : 1;
 		dim3 grid((unsigned)(a.mtiles * a.B * a.Hq)), block(NW * 64);
+		a.fold_half = fold_half_of(a, NW, (int64_t)grid.x, D == 64 || WPS == 2);
 		if (BIAS && a.dbias && a.softcap > 0.f)
-			hipLaunchKernelGGL((bwd_dq_kernel<T, D, NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, false, BIAS, BIAS>), grid, block, 0, s, a);
+			hipLaunchKernelGGL((bwd_dq_kernel<T, D, NW, C::DQ_QB, WPS, BIAS, DROP, false, BIAS, BIAS>), grid, block, 0, s, a);
 		else if (BIAS && a.dbias)
-			hipLaunchKernelGGL((bwd_dq_kernel<T, D, NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, false, false, BIAS>), grid, block, 0, s, a);
+			hipLaunchKernelGGL((bwd_dq_kernel<T, D, NW, C::DQ_QB, WPS, BIAS, DROP, false, false, BIAS>), grid, block, 0, s, a);
 		else if (BIAS && a.softcap > 0.f)
-			hipLaunchKernelGGL((bwd_dq_kernel<T, D, NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, false, BIAS>), grid, block, 0, s, a);
+			hipLaunchKernelGGL((bwd_dq_kernel<T, D, NW, C::DQ_QB, WPS, BIAS, DROP, false, BIAS>), grid, block, 0, s, a);
 		else if (BIAS && a.bias_lds)
-			hipLaunchKernelGGL((bwd_dq_kernel<T, D, NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, BIAS>), grid, block, 0, s, a);
+			hipLaunchKernelGGL((bwd_dq_kernel<T, D, NW, C::DQ_QB, WPS, BIAS, DROP, BIAS>), grid, block, 0, s, a);
 		else
-			hipLaunchKernelGGL((bwd_dq_kernel<T, D, NW, C::DQ_QB, C::DQ_WPS, BIAS, DROP, false>), grid, block, 0, s, a);
+			hipLaunchKernelGGL((bwd_dq_kernel<T, D, NW, C::DQ_QB, WPS, BIAS, DROP, false>), grid, block, 0, s, a);
 	};
 	auto launch_dq = [&]() {
 		if constexpr (C::DQ_NW == 8) {
-			// a grid that leaves at least half of the chip idle: workgroups of 128 rows instead of 256 (see the forward)
+			// a grid that leaves at least half of the chip idle (causal: a grid of up to one 256-row workgroup per CU):
+			// workgroups of 128 rows instead of 256 (see the forward)
 			int64_t wgs = (int64_t)((a.Sq + 127) / 128) * a.B * a.Hq;
-			if (wgs <= kNumCU) return launch_dq_cfg(std::integral_constant<int, 4>{});
+			const bool two_per_cu = a.causal && (int64_t)a.Sk * D * 4 <= (4 << 20);  // (K and V of a head fit an XCD's L2)
+			if (wgs <= kNumCU) return launch_dq_cfg(std::integral_constant<int, 4>{}, std::integral_constant<int, C::DQ_WPS>{});
+			if constexpr (D == 64 || !BIAS) {  // (D = 128 with bias would spill within 256 registers)
+				if (two_per_cu && wgs <= 2 * kNumCU)
+					return launch_dq_cfg(std::integral_constant<int, 4>{}, std::integral_constant<int, (D == 128 ? 2 : 1)>{});
+			}
 		}
-		launch_dq_cfg(std::integral_constant<int, C::DQ_NW>{});
+		launch_dq_cfg(std::integral_constant<int, C::DQ_NW>{}, std::integral_constant<int, C::DQ_WPS>{});
 	};
 	if (fused_delta) launch_dq();
 	if (a.stages & 2) {

@@ -51,7 +51,27 @@ inline int launch_order(const KArgs& a, int heads, int per_xcd, int64_t stream_b
 	return e;
 }
 
+// Workgroup ids of the first half of a causal grid that runs two 4-wave workgroups per CU (see decode_block), else 0.
+// two_per_cu: the kernel variant leaves room for two workgroups on a CU (registers, LDS).  Measured with and without,
+// B2 Hq8 Hkv2 S4096 D128 forward 0.086 / 0.109 ms (unfolded, the two batch rows put their long tiles on the same CUs),
+// a single group B1 Hq8 S8192 0.163 / 0.168 ms.
+inline int fold_half_of(const KArgs& a, int nw, int64_t total, bool two_per_cu) {
+	if (!two_per_cu || nw != 4 || !a.causal || a.win_left >= 0 || a.xcd_remap > 1) return 0;
+	if (total <= kNumCU || total > 2 * kNumCU || total % 16) return 0;
+	return (int)(total / 2);
+}
+
 FA2_DEV void decode_block(const KArgs& a, int& mt, int& h, int& b, int id = (int)blockIdx.x) {
+	if (a.fold_half && id >= a.fold_half) {
+		// A causal grid of two workgroups per CU, all resident at once: the first half of the workgroup ids takes the
+		// first place of every CU, the second half the second place in the same order of CUs.  The first half runs
+		// from the longest tile down; the second half is visited backwards, so that the CU with the longest tile of
+		// the first half gets the shortest of the second (on every XCD for itself when groups are placed by XCD).
+		if (a.xcd_remap)
+			id = (((a.fold_half >> 3) + ((a.fold_half >> 2) - 1 - (id >> 3))) << 3) | (id & 7);
+		else
+			id = a.fold_half + (2 * a.fold_half - 1 - id);
+	}
 	if (a.xcd_remap == 2) {
 		// A bias without a head axis is re-read by every head: one batch per XCD, and on an
 		// XCD the heads of one row tile next to each other, so that the tile of bias they all
@@ -1053,6 +1073,7 @@ hipError_t launch_fwd_cfg(bool bias, bool drop, KArgs& a, hipStream_t s) {
 	a.interleave = a.xcd_remap ? launch_order(a, a.Hq / a.Hkv, groups / 8, (int64_t)a.Sk * D * 4) : 1;
 	if (bias && a.bias_sh == 0 && a.B % 8 == 0) a.xcd_remap = a.kv_lens ? 3 : 2;
 	dim3 grid((unsigned)(a.mtiles * a.B * a.Hq)), block(NW * 64);
+	a.fold_half = fold_half_of(a, NW, (int64_t)grid.x, D == 64 || WPS == 2);
 	const bool blds = bias && a.bias_lds;
 	if (a.softcap > 0.f && drop)
 		hipLaunchKernelGGL((fwd_kernel<T, D, NW, QB, WPS, true, true, false, false, true>), grid, block, 0, s, a);
@@ -1079,9 +1100,18 @@ hipError_t launch_fwd_t(bool bias, bool drop, KArgs& a, hipStream_t s) {
 	typedef FwdCfg<T, D> C;
 	if constexpr (C::NW == 8) {
 		// A grid that leaves at least half of the chip idle (small batch x heads, short sequences): workgroups of
-		// 128 rows instead of 256, twice as many of them, still at most one per CU.
+		// 128 rows instead of 256, twice as many of them, still at most one per CU.  Under a causal mask up to two per
+		// CU: the row tiles differ in length, and 256 workgroups of 256 rows wait for the longest while half of the chip
+		// has run out of work (B1 Hq8 S8192: D = 64 0.154 -> 0.112 ms, D = 128 0.193 -> 0.183 ms; non-causal 0.235 -> 0.339 ms).
+		// Tiles of 128 rows read K and V twice as often: only where the K and V of a head stay in an XCD's L2 (4 MiB;
+		// B1 H4 S16384 D = 128, 8 MiB a head: 0.372 -> 0.568 ms).
 		int64_t wgs = (int64_t)((a.Sq + 127) / 128) * a.B * a.Hq;
+		const bool two_per_cu = a.causal && (int64_t)a.Sk * D * 4 <= (4 << 20);
 		if (wgs <= kNumCU) return launch_fwd_cfg<T, D, 4, 1>(bias, drop, a, s);
+		// (two per CU: at most 256 registers a wave, which D = 64 keeps to anyway; at D = 128 the variants with bias
+		// would spill and stay with 256 rows)
+		if (two_per_cu && wgs <= 2 * kNumCU && (D == 64 || (!bias && !(a.softcap > 0.f))))
+			return launch_fwd_cfg<T, D, 4, (D == 128 ? 2 : 1)>(bias, drop, a, s);
 	}
 	return launch_fwd_cfg<T, D, C::NW, C::WPS>(bias, drop, a, s);
 }

@@ -45,6 +45,7 @@ struct KArgs {
 	// kernel sums, scales and stores them.  1 = no split.
 	int kv_hsplit;
 	float* dkv_part;
+	int fold_half;   // forward / dQ: workgroup ids from this one on are visited backwards (0 = off; see decode_block())
 	int interleave;  // xcd_remap 1: this many (batch, kv-head) groups of an XCD advance through their tiles together (1, 2 or 4)
 	int stages;      // backward: bit 0 delta, bit 1 dK/dV, bit 2 dQ
 	int dq_makes_delta;  // the dQ kernel computes delta itself (and stores it for the dK/dV kernel)

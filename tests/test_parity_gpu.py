@@ -227,9 +227,17 @@ def test_grids_that_fill_the_chip(D, dtype):
 	"""The forward and dQ kernels tile the rows in 128 when that still gives at most one workgroup per CU, which is what
 	the small shapes of the other tests get; these shapes (B x Hq x ceil(Sq / 128) > 256) take the 256-row workgroups
 	with every kind of operand: causal, dropout, bias through LDS and loaded directly (fp32), key lengths, lengths,
-	sliding window, soft-capping with the bias gradient."""
+	sliding window, soft-capping with the bias gradient.  Causal grids of 257 to 512 such units run two 128-row
+	workgroups per CU with the second half of the launch order reversed (B4 Hq16, B3 Hq32, B3 Hq24 below: groups placed
+	by XCD and in plain order), larger ones 256 rows (B4 Hq32)."""
 	B, Hq, Hkv, S = 4, 16, 4, 520
-	assert B * Hq * ((S + 127) // 128) > 256
+	assert 256 < B * Hq * ((S + 127) // 128) <= 512
+	assert 2 * B * Hq * ((S + 127) // 128) > 512
+	_run_case(B, S, S, 2 * Hq, 2 * Hkv, D, dtype, causal=True, data_seed=5)
+	_run_case(B, S, S, 2 * Hq, 2 * Hkv, D, dtype, causal=True, p=0.2, seed=3, data_seed=6)
+	_run_case(3, S, S, 2 * Hq, Hkv, D, dtype, causal=True, seqlens=[520, 1, 300], data_seed=7)
+	_run_case(3, 700, 700, 8, 1, D, dtype, causal=True, data_seed=8)     # 144 units: at most one workgroup per CU, not folded
+	_run_case(3, 700, 700, 24, 3, D, dtype, causal=True, data_seed=9)  # 432 units, groups not a multiple of 8: folded over the plain order
 	_run_case(B, S, S, Hq, Hkv, D, dtype, causal=True)
 	_run_case(B, S, S, Hq, Hkv, D, dtype, causal=True, p=0.2, seed=3, data_seed=1)
 	_run_case(B, S, 456, Hq, Hkv, D, dtype, causal=False, bias_shape=(B, 1, S, 456), data_seed=2)
