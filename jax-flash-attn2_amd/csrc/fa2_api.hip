@@ -210,11 +210,26 @@ static int bwd_step_split(const fa2_params* p) {
 	long steps = (long)(p->Hq / p->Hkv) * ((p->Sq + 127) / 128);  // of the longest key tile, in units of 128 rows
 	long parts = wgs > 0 ? 256 / wgs : 1;  // fill the chip
 	if (p->causal && wgs < 512) {
-		// Causal key tiles differ in length (the first has all the steps, the last one row block's), and with at most
-		// two workgroups per CU the longest sets the time: about 1024 workgroups of at least 64 steps pack well
-		// (B4 Hq32 Hkv2 S4096 D128: dK/dV 1.56 ms unsplit, 1.06 ms in 4 parts; Hkv1 3.00 and 1.07 ms in 8 parts).
-		long bal = (1024 + wgs / 2) / wgs;
-		if (bal > steps / 64) bal = steps / 64;
+		// Causal key tiles differ in length (the first has all the steps, the last one row block's), and with one
+		// workgroup per CU the longest sets the time.  Measured (D = 128, dK/dV kernel): up to 128 workgroups do best in
+		// 8 parts, one per XCD, down to 16 steps a part (B4 Hq32 Hkv1 S4096 3.00 ms unsplit, 1.58 in 2, 1.07 in 8;
+		// B2 Hq8 Hkv2 S4096 0.209 ms in 2, 0.172 in 8); above that about 1024 workgroups of at least 64 steps - up to
+		// 256 workgroups at least 2 parts (B4 Hq32 Hkv2 S4096 1.56 ms unsplit, 1.06 in 2 or 4; B1 Hq32 Hkv8 S4096 0.39 /
+		// 0.27 in 2 / 0.29 in 4; B1 H8 S4096, 32 steps, 0.103 / 0.090 in 2; B3 Hq32 Hkv4, 384 workgroups, 1.53 / 1.05
+		// in 2 / 0.98 in 3; B1 H8 S6144, 384 of 48 steps, 0.163 / 0.185 in 2); from 512 on the launch order packs them
+		// unsplit.
+		long bal;
+		if (wgs <= 128) {
+			bal = steps / 16;
+		} else if (wgs <= 256) {
+			bal = steps / 64 > 2 ? steps / 64 : 2;
+			if (bal > 4) bal = 4;
+			if (bal > steps / 16) bal = steps / 16;
+		} else {
+			bal = (1024 + wgs / 2) / wgs;
+			if (bal > steps / 64) bal = steps / 64;
+		}
+		if (bal > 8) bal = 8;
 		if (bal > parts) parts = bal;
 	}
 	if (parts > 8) parts = 8;

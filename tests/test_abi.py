@@ -219,7 +219,8 @@ def test_backward_split_scratch_only_on_small_grids():
 	assert n == base + 6 * (1 * 2 * 512 * 2 * 64 * 4)
 	assert need(2, 512, 8, 8)[0] == 0          # only 4 steps per key tile: the split would cost more than it saves
 	assert need(1, 100, 2, 2)[0] == 0
-	# causal key tiles differ in length: fewer than 512 workgroups are split further, towards 1024 parts of at least 64 steps
+	# causal key tiles differ in length: fewer than 512 workgroups are split further - up to 128 into 8 parts of at least
+	# 16 steps, more towards 1024 parts of at least 64 steps (but at least 2 parts)
 	n, base = need(1, 4096, 32, 8, causal=1)   # 256 workgroups, 128 steps: 2 parts
 	assert n == base + 2 * (1 * 8 * 4096 * 2 * 128 * 4)
 	n, base = need(4, 4096, 32, 2, causal=1)   # 256 workgroups, 512 steps: 4 parts
@@ -228,6 +229,10 @@ def test_backward_split_scratch_only_on_small_grids():
 	assert n == base + 8 * (4 * 1 * 4096 * 2 * 128 * 4)
 	n, base = need(3, 4096, 32, 4, causal=1)   # 384 workgroups: 3 parts
 	assert n == base + 3 * (3 * 4 * 4096 * 2 * 128 * 4)
+	n, base = need(2, 4096, 8, 2, causal=1)    # 128 workgroups, 128 steps: 8 parts of 16 steps
+	assert n == base + 8 * (2 * 2 * 4096 * 2 * 128 * 4)
+	n, base = need(1, 4096, 8, 8, causal=1)    # 256 workgroups, 32 steps: 2 parts
+	assert n == base + 2 * (1 * 8 * 4096 * 2 * 128 * 4)
 	assert need(2, 4096, 32, 8, causal=1)[0] == 0   # 512 workgroups pack well unsplit
 	assert need(4, 4096, 32, 8, causal=1)[0] == 0
 	n, base = need(1, 2048, 8, 8, causal=1)    # 16 steps: the 2 parts that fill the chip, no more
