@@ -1027,8 +1027,8 @@ template <typename T, int D>
 struct FwdCfg {
 	// D <= 128: 8 waves, two per SIMD (<= 256 registers each): while one waits on LDS or
 	// on a matrix product the other issues.  D = 256 needs the whole register file.
-	// (two independent workgroups of 4 waves per CU instead of one of 8 - so that the waves sharing a SIMD
-	// are not tied to the same barriers - measured the same duration on the 4096-token workload)
+	// (the launcher prefers two independent workgroups of 4 waves per CU where the K and V of a head fit an XCD's L2,
+	// see launch_fwd_t)
 	static constexpr int NW = D <= 128 ? 8 : 4;
 	static constexpr int QB = 1;
 	static constexpr int WPS = 1;
@@ -1100,17 +1100,21 @@ hipError_t launch_fwd_t(bool bias, bool drop, KArgs& a, hipStream_t s) {
 	typedef FwdCfg<T, D> C;
 	if constexpr (C::NW == 8) {
 		// A grid that leaves at least half of the chip idle (small batch x heads, short sequences): workgroups of
-		// 128 rows instead of 256, twice as many of them, still at most one per CU.  Under a causal mask up to two per
-		// CU: the row tiles differ in length, and 256 workgroups of 256 rows wait for the longest while half of the chip
-		// has run out of work (B1 Hq8 S8192: D = 64 0.154 -> 0.112 ms, D = 128 0.193 -> 0.183 ms; non-causal 0.235 -> 0.339 ms).
-		// Tiles of 128 rows read K and V twice as often: only where the K and V of a head stay in an XCD's L2 (4 MiB;
-		// B1 H4 S16384 D = 128, 8 MiB a head: 0.372 -> 0.568 ms).
+		// 128 rows instead of 256, twice as many of them, still at most one per CU.
 		int64_t wgs = (int64_t)((a.Sq + 127) / 128) * a.B * a.Hq;
-		const bool two_per_cu = a.causal && (int64_t)a.Sk * D * 4 <= (4 << 20);
 		if (wgs <= kNumCU) return launch_fwd_cfg<T, D, 4, 1>(bias, drop, a, s);
-		// (two per CU: at most 256 registers a wave, which D = 64 keeps to anyway; at D = 128 the variants with bias
-		// would spill and stay with 256 rows)
-		if (two_per_cu && wgs <= 2 * kNumCU && (D == 64 || (!bias && !(a.softcap > 0.f))))
+		// Larger grids: two independent 128-row workgroups per CU instead of one of 256 rows - the same eight waves, but
+		// one workgroup computes while the other loads its Q, waits for its first tiles or stores its result, and a
+		// causal tile of 128 rows wastes less on the diagonal.  They read K and V twice as often, so only where the K
+		// and V of a head stay in an XCD's L2 (4 MiB; B1 H4 S16384 D = 128, 8 MiB a head: 0.372 -> 0.568 ms).
+		// D = 64 keeps below 256 registers a wave in every variant and gains everywhere (B32 S512 H12 0.053 -> 0.045 ms,
+		// B128 S197 0.071 -> 0.056 ms, B4 S4096 Hq32 causal 0.377 -> 0.330 ms); D = 128 needs an instantiation bound to
+		// 256 registers, which the variants with bias do not fit, and gains under a causal mask only (B8 S2048 0.330 ->
+		// 0.315 ms, B4 S4096 0.563 -> 0.552 ms; non-causal 0.536 -> 0.545 ms).
+		// (D = 128 at the limit, S = 8192: a grid of up to two such workgroups per CU still gains - B1 Hq8 0.193 -> 0.163 ms,
+		// the tail of 256 long workgroups is what costs there - a larger one does not, B2 Hq32 0.953 -> 0.971 ms)
+		const bool fits_l2 = (int64_t)a.Sk * D * 4 <= ((D == 128 && wgs > 2 * kNumCU) ? (2 << 20) : (4 << 20));
+		if (fits_l2 && (D == 64 || (a.causal && !bias && !(a.softcap > 0.f))))
 			return launch_fwd_cfg<T, D, 4, (D == 128 ? 2 : 1)>(bias, drop, a, s);
 	}
 	return launch_fwd_cfg<T, D, C::NW, C::WPS>(bias, drop, a, s);

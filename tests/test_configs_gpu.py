@@ -129,3 +129,27 @@ def test_c5_dropout_wide_heads_bf16_causal_fwd_bwd():
 	# LSE does not depend on dropout (up to fp32 rounding: the two variants of the kernel hold different running references)
 	_, lse0 = op.fwd(q, k, v, causal=True)
 	assert torch.allclose(lse, lse0, rtol=0, atol=1e-5)
+
+
+@pytest.mark.parametrize("D,S,P,Hq,Hkv", [(64, 16640, 8192, 4, 2), (128, 8448, 4096, 8, 2), (128, 4096, 2048, 32, 8)])
+def test_long_causal_rows_reproduce_their_prefix(D, S, P, Hq, Hkv):
+	"""The forward and dQ kernels run as 128-row workgroups, two per CU, while the K and V of a head fit an XCD's L2, and
+	as 256-row workgroups beyond (the first two shapes; the third stays within).  Out of the oracle's reach at these
+	lengths, but under a causal mask the first P rows of O, LSE and dQ depend on the first P rows and keys only: they
+	must agree with the problem cut to P, which takes the other tiling."""
+	dtype = torch.bfloat16
+	q, k, v = _gen((1, S, Hq, D), 0, 0.5, dtype), _gen((1, S, Hkv, D), 1, 0.5, dtype), _gen((1, S, Hkv, D), 2, 0.5, dtype)
+	do = _gen((1, S, Hq, D), 3, 1.0, dtype)
+	o, lse = op.fwd(q, k, v, causal=True)
+	dq, dk, dv = op.bwd(q, k, v, o, lse, do, causal=True)
+	qp, kp, vp, dop = (t[:, :P].contiguous() for t in (q, k, v, do))
+	o_p, lse_p = op.fwd(qp, kp, vp, causal=True)
+	dq_p, _, _ = op.bwd(qp, kp, vp, o_p, lse_p, dop, causal=True)
+	assert (o[:, :P].float() - o_p.float()).abs().max().item() <= TOL_O[dtype]
+	assert (lse[:, :, :P] - lse_p).abs().max().item() <= 2e-3
+	rel = float((dq[:, :P].float() - dq_p.float()).norm() / dq_p.float().norm())
+	assert rel <= TOL_GRAD_REL_L2, rel
+	o1, _ = op.fwd(q, k, torch.ones_like(v), causal=True)
+	assert (o1.float() - 1).abs().max().item() <= 1e-2
+	for t in (dq, dk, dv):
+		assert torch.isfinite(t.float()).all()
