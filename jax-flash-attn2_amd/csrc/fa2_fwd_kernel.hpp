@@ -1109,12 +1109,13 @@ hipError_t launch_fwd_t(bool bias, bool drop, KArgs& a, hipStream_t s) {
 		// and V of a head stay in an XCD's L2 (4 MiB; B1 H4 S16384 D = 128, 8 MiB a head: 0.372 -> 0.568 ms).
 		// D = 64 keeps below 256 registers a wave in every variant and gains everywhere (B32 S512 H12 0.053 -> 0.045 ms,
 		// B128 S197 0.071 -> 0.056 ms, B4 S4096 Hq32 causal 0.377 -> 0.330 ms); D = 128 needs an instantiation bound to
-		// 256 registers, which the variants with bias do not fit, and gains under a causal mask only (B8 S2048 0.330 ->
-		// 0.315 ms, B4 S4096 0.563 -> 0.552 ms; non-causal 0.536 -> 0.545 ms).
+		// 256 registers, which the variants with bias do not fit, and gains under a causal mask (B8 S2048 0.330 -> 0.315 ms,
+		// B4 S4096 0.563 -> 0.552 ms) but not without at 2048 keys (0.536 -> 0.545 ms).
 		// (D = 128 at the limit, S = 8192: a grid of up to two such workgroups per CU still gains - B1 Hq8 0.193 -> 0.163 ms,
 		// the tail of 256 long workgroups is what costs there - a larger one does not, B2 Hq32 0.953 -> 0.971 ms)
 		const bool fits_l2 = (int64_t)a.Sk * D * 4 <= ((D == 128 && wgs > 2 * kNumCU) ? (2 << 20) : (4 << 20));
-		if (fits_l2 && (D == 64 || (a.causal && !bias && !(a.softcap > 0.f))))
+		// (non-causal D = 128: up to 1024 keys, where the start and end of a workgroup weigh most - B16 S1024 0.316 -> 0.297 ms)
+		if (fits_l2 && (D == 64 || ((a.causal || a.Sk <= 1024) && !bias && !(a.softcap > 0.f))))
 			return launch_fwd_cfg<T, D, 4, (D == 128 ? 2 : 1)>(bias, drop, a, s);
 	}
 	return launch_fwd_cfg<T, D, C::NW, C::WPS>(bias, drop, a, s);
