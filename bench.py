@@ -110,20 +110,30 @@ def mfma_peak(torch, dev):
 	"""What the chip sustains on bf16 matrix products alone (random operands), and at which clock."""
 	import ctypes
 
-	from jax_flash_attn2 import _lib
-
-	lib = _lib.load()
-	wgs, iters = 1024, 4000
-	buf = torch.zeros(16 + wgs * 1024, dtype=torch.uint8, device=dev)
+	# the measurement kernel lives in its own small library beside the product library
+	path = os.path.join(ROOT, "jax-flash-attn2_amd", "libfa2_bench.so")
+	if not os.path.exists(path):
+		return None
+	lib = ctypes.CDLL(path)
+	lib.fa2_bench_mfma.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+	lib.fa2_bench_mfma.restype = ctypes.c_int
+	wgs, iters = 1024, 2000
+	buf = torch.zeros(16 + wgs * 2048, dtype=torch.uint8, device=dev)
 	st = torch.cuda.current_stream(dev).cuda_stream
-	run = lambda n: _lib.check(lib.fa2_bench_mfma(buf.data_ptr(), buf.numel(), wgs, n, st))
+
+	def run(n):
+		rc = lib.fa2_bench_mfma(buf.data_ptr(), buf.numel(), wgs, n, st)
+		if rc:
+			raise RuntimeError(f"fa2_bench_mfma failed ({rc})")
+
 	run(iters)  # settle the clocks
 	torch.cuda.synchronize()
 	ms = event_time_ms(lambda: run(iters), 3, torch)
 	ticks = buf[:16].cpu().view(torch.int64)
-	flops = wgs * 4.0 * iters * 32 * 32768
+	flops = wgs * 8.0 * iters * 32 * 32768
 	return {"tflops": flops / (ms * 1e-3) / 1e12, "clock_mhz": float(ticks[0]) / (float(ticks[1]) / 100.0),
-	        "what": "v_mfma_f32_32x32x16_bf16 only, random operands, 4 waves/CU x 4 independent chains"}
+	        "what": "v_mfma_f32_32x32x16_bf16 only, random operands, 8 waves/CU x 4 chains whose accumulators stay live "
+	                "over the whole loop"}
 
 
 def cpu_baseline(w):
@@ -277,14 +287,25 @@ def main():
 	total = ff * (3.5 if w["bwd"] else 1.0)
 	tflops = total / (ms * 1e-3) / 1e12
 
-	# per-kernel durations, HIP events on the launch stream.  The backward of a step is two launches: the dQ
-	# kernel, which also forms delta (stages 5), then the dK/dV kernel (stages 2); they are timed as launched there.
+	# Per-kernel durations: HIP events on the launch stream, recorded between the launches of whole steps, so each
+	# kernel is timed in the place it has in a step (after the kernel that precedes it there, at the clock the step
+	# runs at).  The backward of a step is two launches: the dQ kernel, which also forms delta (stages 5), then the
+	# dK/dV kernel (stages 2) - together exactly the launches of fa2_bwd.
 	it = max(3, min(args.steps, 20))
-	kern = {"fwd": event_time_ms(plan.forward, it, torch)}
+	names = ["fwd", "bwd_dq", "bwd_dkdv"] if w["bwd"] else ["fwd"]
+	calls = {"fwd": plan.forward, "bwd_dq": lambda: plan.backward(5), "bwd_dkdv": lambda: plan.backward(2)}
+	evs = [[torch.cuda.Event(enable_timing=True) for _ in range(len(names) + 1)] for _ in range(it)]
+	for _ in range(2):
+		step()
+	for e in evs:
+		e[0].record()
+		for i, n in enumerate(names):
+			calls[n]()
+			e[i + 1].record()
+	torch.cuda.synchronize()
+	kern = {n: sum(e[i].elapsed_time(e[i + 1]) for e in evs) / it for i, n in enumerate(names)}
 	alg = {"fwd": ff}
 	if w["bwd"]:
-		kern["bwd_dq"] = event_time_ms(lambda: plan.backward(5), it, torch)
-		kern["bwd_dkdv"] = event_time_ms(lambda: plan.backward(2), it, torch)
 		# 5-product convention: S, dP, dV, dK belong to the dK/dV kernel (4 x 0.5 fwd), dQ to the dQ kernel;
 		# the dQ kernel's recomputation of S and dP is not counted.
 		alg["bwd_dkdv"] = 2.0 * ff
@@ -342,8 +363,9 @@ def main():
 		                        "what": "same launches, q = k = v = dO = 0 (identical instruction stream and traffic)"}
 	if not args.no_mfma_peak:
 		mp = mfma_peak(torch, dev)
-		out["mfma_peak_measured"] = mp
-		roofline["frac_of_measured_peak"] = achieved / mp["tflops"]
+		if mp is not None:
+			out["mfma_peak_measured"] = mp
+			roofline["frac_of_measured_peak"] = achieved / mp["tflops"]
 	if not args.no_cpu_baseline:
 		out["cpu_baseline"] = cpu_baseline(w)
 	print(json.dumps(out))

@@ -69,7 +69,9 @@ typedef struct fa2_params {
 	                           (_forward_triton.py:127-132)                */
 	float scale;            /* softmax scale, must be > 0; applied to the fp32 result of q.k^T,
 	                           as the reference does (_forward_triton.py:281)  */
-	float p_drop;           /* dropout probability in [0,1)                */
+	float p_drop;           /* dropout probability in [0,1); realised in steps of 2^-16: an element is dropped
+	                           with probability floor(p_drop * 65536) / 65536 and kept values are scaled by the
+	                           reciprocal of the realised keep probability, so E[O] is exact (see fa2_dropout_mask) */
 	uint64_t seed;          /* Philox key for the dropout keep-mask        */
 
 	fa2_tensor q, k, v, o;  /* o is written by fa2_fwd, read by fa2_bwd    */
@@ -117,7 +119,13 @@ typedef struct fa2_params {
 	const uint64_t* seed_dev;
 
 	/* Optional per-batch number of valid KEYS: keys j >= kv_lens[b] are masked, query rows
-	 * are not touched and causal stays aligned to the full Sk.  Unlike `seqlens` it may be
+	 * are not touched and causal / window stay aligned to the FULL Sk (row i is aligned with key i + Sk - Sq).
+	 * This differs on purpose from the key_padding_mask of the reference's naive attention, which aligns its
+	 * window to the number of valid keys (refrence_call.py:58-66): kv_lens describes padding at the end of a
+	 * key axis whose positions keep their meaning (a KV cache, a bias that is indexed by absolute key), so
+	 * shortening a batch row must not shift which keys a query row may see.  Callers that want the other
+	 * alignment shift `window_left / window_right` by Sk - kv_len themselves (one batch row per call), or use
+	 * `seqlens`, which shortens both axes.  Unlike `seqlens` it may be
 	 * combined with a bias and with Sq != Sk (key padding of cross attention, or of a
 	 * batch that also carries a bias); key tiles beyond the length are skipped, not
 	 * masked.  A row left without any allowed key gives O = 0 and lse = -inf.       */
@@ -137,15 +145,20 @@ typedef struct fa2_params {
 	float softcap;
 
 	/* Optional gradient of the additive bias (backward only; requires `bias` or `softcap`, i.e. the kernel
-	 * variants that carry an additive term).  fp32 [B, Hq, Sq, Sk] with the element strides given, unit
-	 * stride on Sk, 16-byte aligned with strides that are multiples of 4: receives, per (batch, q-head),
-	 *   dbias[b, h, i, j] = P[i, j] * (dP[i, j] - delta[i]),
-	 * the gradient with respect to the term added to the score (before the softmax scale reaches dQ / dK and
-	 * before the 1 - tanh^2 factor of soft-capping).  A bias that is broadcast over batch or heads has the
-	 * sum of these entries over the broadcast axes as its gradient; that reduction is the caller's (one
-	 * `sum`), so the kernel needs no atomics and stays deterministic.  The dQ kernel writes it, tile by tile:
-	 * positions of key tiles it skips (beyond a length, outside the window or the causal range) are not
-	 * written - pass a zero-filled buffer.  The reference returns no gradient for its bias
+	 * variants that carry an additive term).  fp32, element strides as given, unit stride on Sk, 16-byte aligned
+	 * with strides that are multiples of 4.  The dQ kernel adds, per (batch b, q-head h),
+	 *   P[i, j] * (dP[i, j] - delta[i])
+	 * - the gradient with respect to the term added to the score (before the softmax scale reaches dQ / dK and
+	 * before the 1 - tanh^2 factor of soft-capping) - to dbias[b, h', i, j], h' = h, or h / (Hq / Hkv) when
+	 * bias_group is set.  Two layouts:
+	 *   - one entry per (batch, q-head): [B, Hq, Sq, Sk] with non-zero batch and head strides.  Plain stores,
+	 *     deterministic; B * Hq * Sq * Sk * 4 bytes.
+	 *   - the shape of a broadcast bias: stride 0 on the batch and / or head axis, or Hkv heads with bias_group.
+	 *     Entries shared by several (batch, q-head) pairs are accumulated with hardware fp32 atomic adds, so the
+	 *     buffer is as small as the bias but the order of the additions - the last bits of the sums - is not fixed
+	 *     from run to run, and the adds run at about 0.34 T adds/s.
+	 * Positions of key tiles the kernel skips (beyond a length, outside the window or the causal range) are not
+	 * touched: pass a zero-filled buffer in both layouts.  The reference returns no gradient for its bias
 	 * (_flash_attention.py:88), so this has no counterpart there. */
 	float* dbias;
 	int64_t dbias_stride_b, dbias_stride_h, dbias_stride_m;
@@ -222,13 +235,6 @@ int fa2_dropout_mask(const fa2_params* p, uint8_t* keep, void* hip_stream);
 /* Validate params exactly as fa2_fwd / fa2_bwd would, without launching
  * (host-only; usable without a GPU).  which: 0 = forward, 1 = backward. */
 int fa2_validate(const fa2_params* p, int which);
-
-/* Measurement aid (no counterpart in the reference): launches `workgroups` workgroups of 4 waves
- * that each run `iters` x 32 v_mfma_f32_32x32x16_bf16 on random operands and nothing else.
- * FLOPs = workgroups * 4 * iters * 32 * 32768; the caller times the launch.  scratch (device,
- * >= 16 + workgroups * 1024 bytes): on completion its first two uint64 hold workgroup 0's
- * shader-clock cycles and 100 MHz wall-clock ticks, i.e. the clock the chip sustained. */
-int fa2_bench_mfma(void* scratch, size_t scratch_bytes, int workgroups, int iters, void* hip_stream);
 
 const char* fa2_strerror(int code);
 int fa2_version(void);

@@ -52,6 +52,13 @@ KTensor conv(const fa2_tensor& t) {
 	return k;
 }
 
+// delta [B, Hq, Sq] fp32, rounded up to 256 bytes (p: a completed block)
+size_t bwd_scratch_bytes(const fa2_params* p) {
+	if (p->B <= 0 || p->Hq <= 0 || p->Sq <= 0) return 0;
+	size_t n = (size_t)p->B * (size_t)p->Hq * (size_t)p->Sq * sizeof(float);
+	return (n + 255) & ~(size_t)255;
+}
+
 // own_scratch: the backward brings its scratch itself (fa2_bwd_static), p->scratch is not looked at
 int validate(const fa2_params* p, int which, bool own_scratch = false) {
 	if (!p) return FA2_EINVAL_STRUCT;
@@ -91,7 +98,7 @@ int validate(const fa2_params* p, int which, bool own_scratch = false) {
 			if (p->dbias_stride_b < 0 || p->dbias_stride_h < 0 || p->dbias_stride_m < p->Sk) return FA2_EINVAL_BIAS;
 			if (p->dbias_stride_b % 4 || p->dbias_stride_h % 4 || p->dbias_stride_m % 4) return FA2_EINVAL_BIAS;
 		}
-		size_t need = fa2_bwd_scratch_bytes(p);
+		size_t need = bwd_scratch_bytes(p);
 		if (own_scratch) {
 			if (need > FA2_STATIC_SCRATCH_BYTES) return FA2_ESCRATCH_STATIC;
 		} else if (!p->scratch || ((uintptr_t)p->scratch & 255) || p->scratch_bytes < need) {
@@ -155,7 +162,9 @@ void fill(const fa2_params* p, KArgs& a) {
 	a.drop_k1 = (uint32_t)(p->seed >> 32);
 	a.seed_dev = (const uint32_t*)p->seed_dev;  // little-endian: low word first
 	a.drop_thr = drop_threshold(p->p_drop);
-	a.drop_inv_keep = 1.0f / (1.0f - p->p_drop);
+	// kept values are scaled by the reciprocal of the probability the 16-bit threshold really gives,
+	// (65536 - thr) / 65536, so that the expectation of the output is exact for every p
+	a.drop_inv_keep = 65536.0f / (float)(65536u - a.drop_thr);
 }
 
 }  // namespace
@@ -194,11 +203,9 @@ int fa2_validate(const fa2_params* p, int which) {
 }
 
 size_t fa2_bwd_scratch_bytes(const fa2_params* p) {
-	if (!p || p->struct_size < FA2_PARAMS_SIZE_V1) return 0;
-	if (p->B <= 0 || p->Hq <= 0 || p->Sq <= 0) return 0;
-	// delta [B, Hq, Sq] fp32, rounded up to 256 bytes
-	size_t n = (size_t)p->B * (size_t)p->Hq * (size_t)p->Sq * sizeof(float);
-	return (n + 255) & ~(size_t)255;
+	fa2_params lp;
+	p = complete(p, lp);
+	return p ? bwd_scratch_bytes(p) : 0;
 }
 
 // dK/dV on a small grid: B * Hkv * ceil(Sk / 128) workgroups that leave at least half of the chip idle - the steps a
@@ -245,7 +252,10 @@ static size_t bwd_split_part_bytes(const fa2_params* p, int hs) {
 }
 
 size_t fa2_bwd_split_scratch_bytes(const fa2_params* p) {
-	size_t base = fa2_bwd_scratch_bytes(p);
+	fa2_params lp;
+	p = complete(p, lp);
+	if (!p) return 0;
+	size_t base = bwd_scratch_bytes(p);
 	if (!base || p->Sk <= 0 || p->D <= 0) return 0;
 	int hs = bwd_step_split(p);
 	return hs > 1 ? base + bwd_split_part_bytes(p, hs) : 0;
@@ -278,14 +288,22 @@ static int fwd_split_plan(const fa2_params* p, int* split_len) {
 	return (tiles + per - 1) / per;
 }
 
-size_t fa2_fwd_scratch_bytes(const fa2_params* p) {
-	if (!p || p->struct_size < FA2_PARAMS_SIZE_V1) return 0;
+// p: a completed block.  The split forward knows no window and no soft-capping: such calls run unsplit and
+// need no scratch (the same predicate decides the launch in fa2_fwd).
+static size_t fwd_scratch_bytes(const fa2_params* p) {
 	if (p->B <= 0 || p->Hq <= 0 || p->Sq <= 0 || p->Sk <= 0 || p->D <= 0) return 0;
+	if (p->has_window || p->softcap > 0.f) return 0;
 	int len;
 	int n = fwd_split_plan(p, &len);
 	if (n <= 1) return 0;
 	size_t rows = (size_t)n * (size_t)p->B * (size_t)p->Hq * (size_t)p->Sq;
 	return (rows * ((size_t)p->D + 1) * sizeof(float) + 255) & ~(size_t)255;
+}
+
+size_t fa2_fwd_scratch_bytes(const fa2_params* p) {
+	fa2_params lp;
+	p = complete(p, lp);
+	return p ? fwd_scratch_bytes(p) : 0;
 }
 
 int fa2_fwd(const fa2_params* p, void* hip_stream) {
@@ -296,7 +314,7 @@ int fa2_fwd(const fa2_params* p, void* hip_stream) {
 	KArgs a;
 	fill(p, a);
 	// optional scratch: with enough of it a short query over many keys runs split over key ranges
-	size_t need = (p->has_window || p->softcap > 0.f) ? 0 : fa2_fwd_scratch_bytes(p);  // (the split forward knows no window or soft-capping)
+	size_t need = fwd_scratch_bytes(p);
 	if (need && p->scratch && ((uintptr_t)p->scratch & 255) == 0 && p->scratch_bytes >= need) {
 		a.nsplit = fwd_split_plan(p, &a.split_len);
 		a.pack_gqa = fwd_pack_gqa(p) ? 1 : 0;
@@ -319,7 +337,7 @@ static int bwd_launch(const fa2_params* p, void* hip_stream, int stages, void* s
 	a.dkv_part = nullptr;
 	{
 		int hs = bwd_step_split(p);
-		size_t base = fa2_bwd_scratch_bytes(p);
+		size_t base = bwd_scratch_bytes(p);
 		if (hs > 1 && scratch_bytes >= base + bwd_split_part_bytes(p, hs)) {
 			a.kv_hsplit = hs;
 			a.dkv_part = (float*)((char*)scratch_ptr + base);
@@ -334,6 +352,10 @@ static int bwd_launch(const fa2_params* p, void* hip_stream, int stages, void* s
 	a.dbias_sb = p->dbias_stride_b * 4;
 	a.dbias_sh = p->dbias_stride_h * 4;
 	a.dbias_sm = p->dbias_stride_m * 4;
+	a.dbias_atomic = p->dbias && ((p->dbias_stride_b == 0 && p->B > 1) || (p->dbias_stride_h == 0 && p->Hq > 1) ||
+	                              (p->bias_group && p->Hq > p->Hkv))
+	                     ? 1
+	                     : 0;
 	hipError_t e = fa2::launch_bwd(p->dtype, p->D, p->bias != nullptr || p->softcap > 0.f, p->p_drop > 0.f, a, (hipStream_t)hip_stream);
 	return e == hipSuccess ? FA2_OK : FA2_EHIP;
 }

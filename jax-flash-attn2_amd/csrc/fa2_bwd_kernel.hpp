@@ -58,8 +58,17 @@ __global__ __launch_bounds__(256) void bwd_delta_kernel(const KArgs a) {
 // ---------------------------------------------------------------------------
 // BIAS_T: the bias has the element type of q / k / v (no run-time type dispatch per value)
 // CAP: tanh soft-capping of the scores (see the forward kernel); the bias itself may then be absent
-template <typename T, int D, int NW, int QB, bool BIAS, bool DROP, bool BIAS_T, bool CAP = false>
-__global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
+// One key tile `nt` of (batch b, kv-head hk): the whole life of its dK / dV accumulators.  hsi / hsplit: this workgroup's
+// share when the streamed steps of the tile are split over workgroups.  `order`: the order in which the streamed
+// (q-head, query tile) steps are visited -
+//   0  head by head, query tiles ascending inside a head;
+//   1  query tile by query tile ascending, the r q-heads inside a tile (starting with head `rot`);
+//   2  the same with the query tiles descending.
+// With 1 and 2 every workgroup of a KV group that walks in the same direction is at the same query tile at the same
+// time, whatever its key tile - the tiles of Q / dO they stream are then fetched from memory once per XCD.
+template <typename T, int D, int NW, int QB, bool BIAS, bool DROP, bool BIAS_T, bool CAP>
+FA2_DEV void bwd_dkdv_tile(const KArgs& a, const int nt, const int hk, const int b, const int hsi, const int hsplit, const int order,
+                           const int rot) {
 	static_assert(!CAP || (BIAS && !BIAS_T), "soft-capping runs on the plain path with bias");
 	typedef typename T::V8 V8;
 	constexpr int BN = NW * 32;     // keys per workgroup
@@ -116,43 +125,9 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		}
 	}
 
-	// blockIdx.x -> (key tile, kv head, batch); key tiles of one (b, kv head) stay on one XCD
-	// (with the steps of a key tile split over workgroups: the parts of one key tile are adjacent)
-	int nt, hk, b;
-	const int hsplit = a.kv_hsplit > 1 ? a.kv_hsplit : 1;
-	const int hsi = hsplit > 1 ? (int)blockIdx.x % hsplit : 0;
-	{
-		int id = hsplit > 1 ? (int)blockIdx.x / hsplit : (int)blockIdx.x;
-		int per_group = a.mtiles;
-		int grp, within;
-		if (a.xcd_remap >= 2) {
-			// bias shared by the heads: one batch per XCD, the kv-heads of one key tile adjacent
-			int xcd = id & 7, j = id >> 3;
-			int per_batch = per_group * a.Hkv;
-			int rem = j % per_batch;
-			grp = ((j / per_batch) * 8 + xcd) * a.Hkv + rem % a.Hkv;
-			within = rem / a.Hkv;
-			if (a.xcd_remap == 3) {
-				// batch rows of different key lengths: the units (batch, key tile) of one batch go round the XCDs
-				int u = j / a.Hkv, nb8 = a.B >> 3;
-				within = u / nb8;
-				grp = (((xcd - within) & 7) + 8 * (u % nb8)) * a.Hkv + j % a.Hkv;
-			}
-		} else if (a.xcd_remap) {
-			int xcd = id & 7, j = id >> 3;
-			// a.interleave = e groups of an XCD advance together: e adjacent workgroups are the same key tile (see launch_order())
-			int e = a.interleave;
-			int sgi = j / (e * per_group), rem = j % (e * per_group);
-			grp = (sgi * e + rem % e) * 8 + xcd;
-			within = rem / e;
-		} else {
-			grp = id / per_group;
-			within = id % per_group;
-		}
-		hk = grp % a.Hkv;
-		b = grp / a.Hkv;
-		nt = within;  // early key tiles see the most query rows under a causal mask: first
-	}
+	// (a workgroup may handle two key tiles one after the other: the LDS buffers of the previous one are free
+	// once every wave has left its last step)
+	__syncthreads();
 	const int r = a.Hq / a.Hkv;
 
 	int sq_eff = a.Sq, sk_eff = a.Sk;
@@ -246,9 +221,18 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	// one: it is not bound by that traffic, and 32 workgroups asking for the same lines at the same
 	// moment wait on each other.)
 	auto decode_step = [&](int step, int& hq, int& m0) __attribute__((always_inline)) {
-		int hi = step / nq;
+		int hi, i;
+		if (order == 0) {
+			hi = step / nq;
+			i = step - hi * nq;
+		} else {
+			int t = step / r;
+			hi = step - t * r + rot;
+			hi = hi >= r ? hi - r : hi;
+			i = order == 2 ? nq - 1 - t : t;
+		}
 		hq = hk * r + hi;
-		m0 = (q_lo + (step - hi * nq)) * BMQ;
+		m0 = (q_lo + i) * BMQ;
 	};
 	// start the copies of streamed tile `step` (rows beyond Sq are fetched from the last valid row)
 	auto issue_tile = [&](int step, FA2_LDS char* qdst, FA2_LDS char* dodst) __attribute__((always_inline)) {
@@ -807,13 +791,22 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	if (wn0 + 32 > sk_eff) i_diag = nq;  // ragged key block: always masked
 	i_diag = i_diag < 0 ? 0 : (i_diag > nq ? nq : i_diag);
 	i_full = i_full < i_diag ? i_diag : (i_full > nq ? nq : i_full);
-	for (int hi = 0; hi < r && nq > 0; ++hi) {
-		// (each of the three runs clipped to this workgroup's share of the steps)
-		int base = hi * nq;
-		auto clip = [&](int i) { int st = base + i; return st < s_lo ? s_lo : (st > s_hi ? s_hi : st); };
-		for (int st = clip(0); st < clip(i_diag); ++st) run_step(std::true_type{}, st);
-		for (int st = clip(i_diag); st < clip(i_full); ++st) run_step(std::false_type{}, st);
-		for (int st = clip(i_full); st < clip(nq); ++st) run_step(std::true_type{}, st);
+	if (order == 0) {
+		for (int hi = 0; hi < r && nq > 0; ++hi) {
+			// (each of the three runs clipped to this workgroup's share of the steps)
+			int base = hi * nq;
+			auto clip = [&](int i) { int st = base + i; return st < s_lo ? s_lo : (st > s_hi ? s_hi : st); };
+			for (int st = clip(0); st < clip(i_diag); ++st) run_step(std::true_type{}, st);
+			for (int st = clip(i_diag); st < clip(i_full); ++st) run_step(std::false_type{}, st);
+			for (int st = clip(i_full); st < clip(nq); ++st) run_step(std::true_type{}, st);
+		}
+	} else {
+		// query tiles outermost: the same three runs, r steps per query tile, in the direction of the walk
+		const int pa = (order == 2 ? nq - i_full : i_diag) * r, pb = (order == 2 ? nq - i_diag : i_full) * r;
+		auto clip = [&](int st) { return st < s_lo ? s_lo : (st > s_hi ? s_hi : st); };
+		for (int st = clip(0); st < clip(pa); ++st) run_step(std::true_type{}, st);
+		for (int st = clip(pa); st < clip(pb); ++st) run_step(std::false_type{}, st);
+		for (int st = clip(pb); st < clip(steps); ++st) run_step(std::true_type{}, st);
 	}
 
 	// the last matrix products (issued as inline assembly) must have written dk / dv
@@ -851,6 +844,71 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 				            pack2<typename T::V2>(dv[db][4 * aa + 2] * vs_, dv[db][4 * aa + 3] * vs_)};
 				*(u32x2*)(dvp + d0 * 2) = pv;
 			}
+	}
+}
+
+// blockIdx.x -> (key tile or pair of key tiles, kv head, batch); the key tiles of one (b, kv head) stay on one XCD.
+// BIAS_T: the bias has the element type of q / k / v (no run-time type dispatch per value)
+// CAP: tanh soft-capping of the scores (see the forward kernel); the bias itself may then be absent
+template <typename T, int D, int NW, int QB, bool BIAS, bool DROP, bool BIAS_T, bool CAP = false>
+__global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
+	// (with the steps of a key tile split over workgroups: the parts of one key tile are adjacent)
+	int hk, b, within;
+	const int hsplit = a.kv_hsplit > 1 ? a.kv_hsplit : 1;
+	const int hsi = hsplit > 1 ? (int)blockIdx.x % hsplit : 0;
+	{
+		int id = hsplit > 1 ? (int)blockIdx.x / hsplit : (int)blockIdx.x;
+		int per_group = a.mtiles;
+		int grp;
+		if (a.xcd_remap >= 2) {
+			// bias shared by the heads: one batch per XCD, the kv-heads of one key tile adjacent
+			int xcd = id & 7, j = id >> 3;
+			int per_batch = per_group * a.Hkv;
+			int rem = j % per_batch;
+			grp = ((j / per_batch) * 8 + xcd) * a.Hkv + rem % a.Hkv;
+			within = rem / a.Hkv;
+			if (a.xcd_remap == 3) {
+				// batch rows of different key lengths: the units (batch, key tile) of one batch go round the XCDs
+				int u = j / a.Hkv, nb8 = a.B >> 3;
+				within = u / nb8;
+				grp = (((xcd - within) & 7) + 8 * (u % nb8)) * a.Hkv + j % a.Hkv;
+			}
+		} else if (a.xcd_remap) {
+			int xcd = id & 7, j = id >> 3;
+			// a.interleave = e groups of an XCD advance together: e adjacent workgroups are the same key tile (see launch_order())
+			int e = a.interleave;
+			int sgi = j / (e * per_group), rem = j % (e * per_group);
+			grp = (sgi * e + rem % e) * 8 + xcd;
+			within = rem / e;
+		} else {
+			grp = id / per_group;
+			within = id % per_group;
+		}
+		hk = grp % a.Hkv;
+		b = grp / a.Hkv;
+	}
+	const int r = a.Hq / a.Hkv;
+	// (head dim 256 sits at the edge of the register file: it keeps the one walk, as a compile-time constant)
+	constexpr bool WALKS = D <= 128;
+	if constexpr (!WALKS) {
+		bwd_dkdv_tile<T, D, NW, QB, BIAS, DROP, BIAS_T, CAP>(a, within, hk, b, hsi, hsplit, 0, 0);
+	} else if (a.kv_pair) {
+		// Causal self-attention: key tile p streams every query tile from p up, so a workgroup takes tile p and tile
+		// ntiles - 1 - p one after the other - every workgroup then has the same number of steps (no CU waits for the
+		// longest tile, no gaps in the dispatch), and the two walks are arranged so that all workgroups of a KV group
+		// stay together: the long tile runs from the last query tile DOWN (all workgroups start at the same tile and
+		// drop out one by one), the short tile from its diagonal UP (a workgroup that has finished tile p, one step
+		// later than the workgroup of p + 1, joins that workgroup's second walk exactly where it is now).  At any
+		// time the KV group reads two fronts of Q / dO tiles, not one per workgroup.
+		const int ntiles = a.kv_ntiles;
+		const int rot = within % r;
+		// (an odd number of tiles: the middle one is its own partner)
+		const int npass = ntiles - 1 - within == within ? 1 : 2;
+		for (int pass = 0; pass < npass; ++pass)
+			bwd_dkdv_tile<T, D, NW, QB, BIAS, DROP, BIAS_T, CAP>(a, pass == 0 ? within : ntiles - 1 - within, hk, b, 0, 1, pass == 0 ? 2 : 1, rot);
+	} else {
+		// early key tiles see the most query rows under a causal mask: first
+		bwd_dkdv_tile<T, D, NW, QB, BIAS, DROP, BIAS_T, CAP>(a, within, hk, b, hsi, hsplit, a.kv_order, a.kv_order ? within % r : 0);
 	}
 }
 
@@ -1141,6 +1199,9 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 #pragma unroll
 				for (int i = 0; i < 16; ++i) s[qb][i] = dp[qb][i] = 0.f;
 			__builtin_amdgcn_sched_barrier(0);
+#if FA2_SETPRIO
+			__builtin_amdgcn_s_setprio(FA2_SETPRIO);
+#endif
 #pragma unroll
 			for (int ks = 0; ks < KS; ++ks) {
 				V8 ka = *(const FA2_LDS V8*)(lds + koff[ks % KR] + (ks / KR) * 256 + kb * (32 * D * 2));
@@ -1162,6 +1223,9 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 				__builtin_amdgcn_sched_group_barrier(0x008, PF * QB, 0);
 			}
 			__builtin_amdgcn_sched_barrier(0);
+#if FA2_SETPRIO
+			__builtin_amdgcn_s_setprio(0);
+#endif
 			// K^T fragments for dQ^T += K^T dS^T, issued ahead of the elementwise math
 			constexpr bool BOTH_EARLY = DB <= 4;
 			u32x4 kfr[2][DB];
@@ -1205,8 +1269,15 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 						{
 							int j0 = n0 + 32 * kb + 8 * aa + 4 * g;
 							if (qrow[qb] < a.Sq && j0 < a.Sk) {
-								char* dp_ = a.dbias + (int64_t)b * a.dbias_sb + (int64_t)h * a.dbias_sh + (int64_t)qrow[qb] * a.dbias_sm + (int64_t)j0 * 4;
-								if (j0 + 3 < a.Sk) {
+								// (a gradient buffer in the shape of a bias with Hkv heads is indexed like that bias)
+								const int hb = a.bias_group ? hk : h;
+								char* dp_ = a.dbias + (int64_t)b * a.dbias_sb + (int64_t)hb * a.dbias_sh + (int64_t)qrow[qb] * a.dbias_sm + (int64_t)j0 * 4;
+								if (a.dbias_atomic) {
+									// several (batch, q-head) pairs share the entry (broadcast axis of the bias): hardware fp32 adds
+#pragma unroll
+									for (int e = 0; e < 4; ++e)
+										if (j0 + e < a.Sk) unsafeAtomicAdd((float*)dp_ + e, s[qb][4 * aa + e]);
+								} else if (j0 + 3 < a.Sk) {
 									*(f32x4*)dp_ = f32x4{s[qb][4 * aa], s[qb][4 * aa + 1], s[qb][4 * aa + 2], s[qb][4 * aa + 3]};
 								} else {
 #pragma unroll
@@ -1229,6 +1300,9 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 				}
 			}
 			// dQ^T += K^T dS^T
+#if FA2_SETPRIO
+			__builtin_amdgcn_s_setprio(FA2_SETPRIO);
+#endif
 #pragma unroll
 			for (int hf = 0; hf < 2; ++hf) {
 				if (hf == 0 && !BOTH_EARLY) issue_k(1, kfr[1]);
@@ -1237,6 +1311,9 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 #pragma unroll
 					for (int qb = 0; qb < QB; ++qb) dq[qb][db] = mfma32(as_frag<T>(kfr[hf][db]), dsf[qb][hf], dq[qb][db]);
 			}
+#if FA2_SETPRIO
+			__builtin_amdgcn_s_setprio(0);
+#endif
 		}
 	};
 
@@ -1506,6 +1583,23 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 		a.mtiles = (a.Sk + C::KV_BN - 1) / C::KV_BN;
 		a.interleave = a.xcd_remap == 1 ? launch_order(a, 1, groups / 8, (int64_t)(a.Hq / a.Hkv) * a.Sq * D * 4) : 1;
 		const int hs = a.kv_hsplit > 1 ? a.kv_hsplit : 1;
+		// Causal self-attention on a grid that fills the chip in whole rounds: every workgroup takes the key tiles p and
+		// ntiles - 1 - p one after the other (see bwd_dkdv_kernel).  Measured on the 4096-token workload (B4 Hq32 Hkv8):
+		// dK/dV kernel 1.032 -> 1.000 ms and 1318 -> 437 MiB fetched from memory (324 MiB of operands); on the
+		// 32768-token one 31.7 -> 30.3 ms and 87 -> 4.8 GiB (1.14 GiB of operands).  Walking the query tiles outermost
+		// WITHOUT the pairing (kv_order 1 / 2 on one tile per workgroup) measured slower than head by head: 1.065 /
+		// 1.051 ms, so everything else keeps that order.
+		a.kv_order = 0;
+		a.kv_pair = 0;
+		a.kv_ntiles = a.mtiles;
+		if (D <= 128 && hs == 1 && a.causal && a.win_left < 0 && a.Sq == a.Sk && !a.seqlens && !a.kv_lens && a.xcd_remap <= 1 && a.mtiles >= 2) {
+			const int64_t pairs = (int64_t)((a.mtiles + 1) / 2) * groups;
+			if (pairs % kNumCU == 0 || pairs >= 8 * kNumCU) {
+				a.kv_pair = 1;
+				a.mtiles = (a.mtiles + 1) / 2;
+				a.interleave = 1;
+			}
+		}
 		dim3 grid((unsigned)(a.mtiles * a.B * a.Hkv * hs)), block(C::KV_NW * 64);
 		// typed variant: bias in the element type of q, staged through LDS: it also needs 16-byte aligned rows of whole 16-byte pieces
 		bool typed = BIAS && a.bias_dtype == (std::is_same<T, BF16>::value ? 2 : 1);

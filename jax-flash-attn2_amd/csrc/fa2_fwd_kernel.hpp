@@ -20,6 +20,11 @@
 
 namespace fa2 {
 
+// experiment switch: wave priority raised around the clusters of matrix products (0 = off)
+#ifndef FA2_SETPRIO
+#define FA2_SETPRIO 0
+#endif
+
 constexpr int kFwdBN = 64;
 // with bias: the running row maximum is only raised when exceeded by more than this (log2 units)
 constexpr float kRescaleSlack = 8.f;
@@ -495,7 +500,13 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 
 		// online softmax, one query row per lane
 		V8 pf[QB][BN / 16];
+#if FA2_SETPRIO
+		__builtin_amdgcn_s_setprio(FA2_SETPRIO);
+#endif
 		compute_s();
+#if FA2_SETPRIO
+		__builtin_amdgcn_s_setprio(0);
+#endif
 		issue_v(std::integral_constant<int, 0>{}, vfr[0]);
 		// packs P (held in s) to the B operand of the second product
 		auto pack_p = [&](int qb) __attribute__((always_inline)) {
@@ -698,6 +709,9 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 			}
 		};
 		__builtin_amdgcn_sched_barrier(0);
+#if FA2_SETPRIO
+		__builtin_amdgcn_s_setprio(FA2_SETPRIO);
+#endif
 		static_for<0, NBATCH>(pv_batch);
 		// issue order: every product of a batch but the last is followed by the two transposed reads
 		// of one fragment of the next batch (left to itself the compiler's order, and with it the
@@ -709,6 +723,9 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 		}
 		__builtin_amdgcn_sched_group_barrier(0x008, NF * QB, 0);
 		__builtin_amdgcn_sched_barrier(0);
+#if FA2_SETPRIO
+		__builtin_amdgcn_s_setprio(0);
+#endif
 	};
 
 	// Head dim 256 runs one wave per SIMD, so the softmax overlaps the matrix products only if the wave interleaves

@@ -25,6 +25,7 @@ struct KArgs {
 	int bias_lds;    // bias tiles may be copied global->LDS in 16-byte pieces (see fa2_api.hip)
 	char* dbias;     // backward, optional: fp32 [B, Hq, Sq, Sk] gradient of the additive term (dQ kernel variants with bias)
 	int64_t dbias_sb, dbias_sh, dbias_sm;  // bytes
+	int dbias_atomic;  // entries of dbias are shared by several (batch, q-head) pairs (stride 0 on an axis, or Hkv heads): accumulate with atomic adds
 	const int32_t* seqlens;
 	const int32_t* kv_lens;  // [B]: keys at or beyond kv_lens[b] are masked (query rows unaffected)
 	int B, Sq, Sk, Hq, Hkv;
@@ -45,6 +46,10 @@ struct KArgs {
 	// kernel sums, scales and stores them.  1 = no split.
 	int kv_hsplit;
 	float* dkv_part;
+	// dK/dV kernel: order in which a key tile visits its (q-head, query tile) steps (see bwd_dkdv_tile), and whether a
+	// workgroup takes the key tiles p and ntiles - 1 - p one after the other (causal self-attention; a.mtiles then
+	// counts pairs)
+	int kv_order, kv_pair, kv_ntiles;  // kv_ntiles: key tiles per (batch, kv-head)
 	int fold_half;   // forward / dQ: workgroup ids from this one on are visited backwards (0 = off; see decode_block())
 	int interleave;  // xcd_remap 1: this many (batch, kv-head) groups of an XCD advance through their tiles together (1, 2 or 4)
 	int stages;      // backward: bit 0 delta, bit 1 dK/dV, bit 2 dQ

@@ -175,7 +175,8 @@ def fwd(q, k, v, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, 
 def bwd(q, k, v, out, lse, dout, bias=None, seqlens=None, softmax_scale=None, dropout_prob=0.0, causal=False,
         dropout_seed=None, kv_lens=None, window=None, softcap=0.0, need_dbias=False):
 	"""Returns (dq, dk, dv) in the dtypes of q, k, v; dk/dv summed over each KV group.  With `need_dbias` a fourth
-	result: the gradient of the additive bias, fp32, in the shape of `bias` (summed over the axes it is broadcast on)."""
+	result: the gradient of the additive bias, fp32, in the shape of `bias` (summed over the axes it is broadcast on;
+	those sums are atomic adds in the dQ kernel - see fa2_params.dbias - so the buffer is as small as the bias)."""
 	lib = _lib.load()
 	D0 = q.shape[-1]
 	D = _kernel_head_dim(D0)
@@ -200,32 +201,21 @@ def bwd(q, k, v, out, lse, dout, bias=None, seqlens=None, softmax_scale=None, dr
 	if need_dbias:
 		if bias is None or bias.dtype == torch.uint8:
 			raise ValueError("the bias gradient needs a floating-point bias")
-		# the kernel writes the per-(batch, head) gradient and leaves skipped key tiles alone: zero-filled
-		dbias = torch.zeros((B, Hq, Sq, k.shape[1]), dtype=torch.float32, device=q.device)
-		if dbias.shape[3] % 4:  # rows must start on 16 bytes
-			dbias = torch.zeros((B, Hq, Sq, (k.shape[1] + 3) // 4 * 4), dtype=torch.float32, device=q.device)[..., : k.shape[1]]
+		# fp32, zero-filled (the kernel leaves skipped key tiles alone), in the SHAPE OF THE BIAS: on the axes the bias is
+		# broadcast on (size-1 batch / head axis, Hkv heads) the dQ kernel accumulates with atomic adds, so the memory is
+		# that of the bias itself and not B * Hq * Sq * Sk * 4 bytes.  Rows start on 16 bytes.
+		Skp = (k.shape[1] + 3) // 4 * 4
+		dbias = torch.zeros((bias.shape[0], bias.shape[1], Sq, Skp), dtype=torch.float32, device=q.device)[..., : k.shape[1]]
 		p.dbias = dbias.data_ptr()
-		p.dbias_stride_b, p.dbias_stride_h, p.dbias_stride_m = dbias.stride(0), dbias.stride(1), dbias.stride(2)
+		p.dbias_stride_b = 0 if bias.shape[0] == 1 else dbias.stride(0)
+		p.dbias_stride_h = 0 if bias.shape[1] == 1 else dbias.stride(1)
+		p.dbias_stride_m = dbias.stride(2)
 	_lib.check(lib.fa2_bwd(ctypes.byref(p), _stream_ptr(q.device)))
 	if D != D0:
 		dq, dk, dv = dq[..., :D0], dk[..., :D0], dv[..., :D0]
 	if need_dbias:
-		return dq, dk, dv, _reduce_dbias(dbias, bias.shape, k.shape[2])
+		return dq, dk, dv, dbias
 	return dq, dk, dv
-
-
-def _reduce_dbias(full: torch.Tensor, bias_shape, Hkv: int) -> torch.Tensor:
-	"""[B, Hq, Sq, Sk] per-head gradient -> the shape of the bias: summed over the q-heads of a KV group for a bias
-	with Hkv heads, over all heads / batch rows for a size-1 axis (the axes the kernels broadcast the bias on)."""
-	B, Hq = full.shape[:2]
-	Bb, Hb = bias_shape[0], bias_shape[1]
-	if Hb == 1:
-		full = full.sum(dim=1, keepdim=True)
-	elif Hb != Hq:
-		full = full.reshape(B, Hkv, Hq // Hkv, *full.shape[2:]).sum(dim=2)
-	if Bb == 1 and B != 1:
-		full = full.sum(dim=0, keepdim=True)
-	return full
 
 
 def dropout_mask(B, H, Sq, Sk, dropout_prob, dropout_seed, device) -> torch.Tensor:
@@ -291,26 +281,26 @@ class Plan:
 class _FlashAttentionFn(torch.autograd.Function):
 	"""Differentiation rule; the torch spelling of the reference's
 	`flash_attention_call.defvjp(_jax_fwd_attention_call, _jax_bwd_attention_call)`
-	(_flash_attention.py:119-122).  Returns (dq, dk, dv) and None for everything else - except the bias: where
-	the reference returns None for it (_flash_attention.py:88), a floating-point bias that requires a gradient
-	gets one here."""
+	(_flash_attention.py:119-122).  Returns (dq, dk, dv) and None for everything else, as the reference does
+	(_flash_attention.py:88) - unless the caller asked for the gradient of the bias (`bias_grad=True`)."""
 
 	@staticmethod
-	def forward(ctx, q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens=None, window=None, softcap=0.0):
+	def forward(ctx, q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens=None, window=None, softcap=0.0,
+	            bias_grad=False):
 		out, lse = fwd(q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens, window, softcap)
 		ctx.save_for_backward(q, k, v, bias, seqlens, out, lse, kv_lens)
-		ctx.cfg = (softmax_scale, dropout_prob, causal, dropout_seed, window, softcap)
+		ctx.cfg = (softmax_scale, dropout_prob, causal, dropout_seed, window, softcap, bias_grad)
 		return out
 
 	@staticmethod
 	def backward(ctx, dout):
 		q, k, v, bias, seqlens, out, lse, kv_lens = ctx.saved_tensors
-		softmax_scale, dropout_prob, causal, dropout_seed, window, softcap = ctx.cfg
-		need_dbias = bias is not None and ctx.needs_input_grad[3]
+		softmax_scale, dropout_prob, causal, dropout_seed, window, softcap, bias_grad = ctx.cfg
+		need_dbias = bool(bias_grad) and bias is not None and ctx.needs_input_grad[3]
 		res = bwd(q, k, v, out, lse, dout, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens, window, softcap,
 		          need_dbias=need_dbias)
 		dbias = res[3].to(bias.dtype) if need_dbias else None
-		return res[0], res[1], res[2], dbias, None, None, None, None, None, None, None, None
+		return res[0], res[1], res[2], dbias, None, None, None, None, None, None, None, None, None
 
 
 def flash_attention(
@@ -328,6 +318,7 @@ def flash_attention(
 	kv_lens=None,
 	window_size=None,
 	softcap: float = 0.0,
+	bias_grad: bool = False,
 ):
 	"""Same signature as the reference's `triton_flash_attention`
 	(_flash_attention.py:125-157).  `varlen_mode` is accepted for source
@@ -338,11 +329,17 @@ def flash_attention(
 	(left, right) (keyword only): the sliding window of the reference's naive attention
 	(refrence_call.py:32,55-75); a negative bound is none, causal sets right = 0.  `softcap` > 0
 	(keyword only): scores become softcap * tanh(score / softcap) before bias and masks
-	(refrence_call.py:33,48-51)."""
+	(refrence_call.py:33,48-51).  `bias_grad` (keyword only): also differentiate with respect to a floating-point
+	`bias` that requires a gradient - off by default, as the reference returns no gradient for its bias
+	(_flash_attention.py:88); costs a zero-filled fp32 buffer in the shape of the bias and, where the bias is
+	broadcast over batch or heads, atomic adds in the dQ kernel (summation order not fixed)."""
 	del varlen_mode
+	if bias_grad and attention_mask is not None and attention_mask.dim() == 4:
+		raise ValueError("bias_grad needs a floating-point bias, not a boolean mask")
 	if attention_mask is not None and attention_mask.dim() == 4:
 		assert bias is None, "Attention mask is not supported along with attention bias. Just use bias instead."
 		bias, attention_mask = _mask_operand(attention_mask, q), None
 	check_shapes(q, k, v, bias, attention_mask)
 	seqlens = _seqlens_from_mask(attention_mask, q)
-	return _FlashAttentionFn.apply(q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens, window_size, softcap)
+	return _FlashAttentionFn.apply(q, k, v, bias, seqlens, softmax_scale, dropout_prob, causal, dropout_seed, kv_lens, window_size, softcap,
+	                               bias_grad)

@@ -5,7 +5,8 @@ Takes the place of `jax_flash_attn2/flash_attention_triton/_flash_attention.py:2
 of the reference (`_jax_fwd_attention_call`, `_jax_bwd_attention_call`,
 `flash_attention_call`, `flash_attention`): same argument list, same static
 arguments (softmax_scale, dropout_prob, causal, varlen_mode), same residuals
-(q, k, v, bias, mask, out, lse, seed), gradients for q, k, v only.
+(q, k, v, bias, mask, out, lse, seed), gradients for q, k, v (and, on request, the bias).
+The operand / result / attribute lists of the custom calls are spelled once, in `_ffi_spec.py`.
 
 The FFI handlers live in csrc/fa2_xla_ffi.cc (built into libfa2_xla_ffi.so with
 `make -C csrc ffi XLA_FFI_INCLUDE=$(python -c "import jax; print(jax.ffi.include_dir())")`);
@@ -28,6 +29,7 @@ import jax
 import jax.numpy as jnp
 import numpy as np
 
+from . import _ffi_spec as spec
 from ._checks import check_shapes
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -50,18 +52,52 @@ def _register():
 			"(there is no non-HIP fallback for this path)"
 		)
 	lib = ctypes.CDLL(FFI_LIB_PATH)
-	for name in ("fa2_fwd_ffi", "fa2_bwd_ffi", "fa2_dropout_mask_ffi"):
+	for name in spec.HANDLERS:
 		_ffi.register_ffi_target(name, _ffi.pycapsule(getattr(lib, name)), platform="ROCM")
 	_registered = True
+
+
+def _ffi_call(name, out_types):
+	"""`ffi_call` with a batching rule: under `jax.vmap` the custom call is applied to one slice after the other
+	(always correct; the batch axis of the operator itself is the way to batch for speed)."""
+	try:
+		return _ffi.ffi_call(name, out_types, vmap_method="sequential")
+	except TypeError:  # older jax: no vmap_method
+		return _ffi.ffi_call(name, out_types)
 
 
 def _absent(dtype):
 	return jnp.zeros((0,), dtype)
 
 
-def _prep(q, k, v, bias, attention_mask):
-	"""Shape checks of `_fwd_attention_kernel_call` (_forward_triton.py:474-495); the 2-D
-	right-padded mask becomes one length per batch row instead of a packed layout."""
+class _Cfg(tp.NamedTuple):
+	"""Compile-time constants of a call: hashable, the one non-differentiable argument of the differentiation rule."""
+	scale: float
+	dropout_p: float
+	causal: bool
+	bias_group: bool
+	has_window: bool
+	window_left: int
+	window_right: int
+	softcap: float
+	bias_grad: bool
+
+
+def _attr_dict(cfg: _Cfg):
+	"""Attributes of the custom calls in binding order (spec.ATTRS): compile-time constants only (the seed is an operand)."""
+	conv = {"float": np.float32, "bool": bool, "int32_t": np.int32}
+	return {name: conv[ctype](getattr(cfg, name)) for name, ctype in spec.ATTRS}
+
+
+def _operands(q, k, v, bias, attention_mask, kv_lens):
+	"""Shape checks of `_fwd_attention_kernel_call` (_forward_triton.py:474-495) and the optional operands as the
+	handlers take them.  The 2-D right-padded mask becomes one length per batch row instead of a packed layout; a
+	4-D boolean mask is the `bias` operand itself, one byte per position - the kernels add finfo(dtype).min at
+	masked positions, which is what the bias where(mask, 0, finfo(dtype).min) of README.md:188 would add, without
+	that bias ever being built."""
+	if attention_mask is not None and attention_mask.ndim == 4:
+		assert bias is None, "Attention mask is not supported along with attention bias. Just use bias instead."
+		bias, attention_mask = attention_mask.astype(jnp.bool_), None
 	check_shapes(q, k, v, bias, attention_mask)
 	seqlens = _absent(jnp.int32)
 	if attention_mask is not None:
@@ -70,118 +106,149 @@ def _prep(q, k, v, bias, attention_mask):
 		seqlens = (attention_mask != 0).sum(axis=1, dtype=jnp.int32)
 	bias_group = False
 	if bias is None:
-		bias = _absent(q.dtype)
+		bias_op = _absent(q.dtype)
 	else:
-		if bias.dtype not in (jnp.float16, jnp.bfloat16, jnp.float32):
-			bias = bias.astype(jnp.float32)
+		bias_op = bias
+		if bias_op.dtype not in (jnp.float16, jnp.bfloat16, jnp.float32, jnp.bool_, jnp.uint8, jnp.int8):
+			bias_op = bias_op.astype(jnp.float32)
 		bias_group = bias.shape[1] == k.shape[2] and k.shape[2] != q.shape[2] and bias.shape[1] != 1
-	return bias, seqlens, bias_group
-
-
-def _attrs(q, softmax_scale, dropout_prob, causal, bias_group):
-	"""Attributes of the custom calls: compile-time constants only (the seed is an operand)."""
-	scale = 1.0 / math.sqrt(q.shape[-1]) if softmax_scale is None else softmax_scale
-	return dict(
-		scale=np.float32(scale),
-		dropout_p=np.float32(dropout_prob),
-		causal=bool(causal),
-		bias_group=bool(bias_group),
-	)
+	if kv_lens is None:
+		kv_op = _absent(jnp.int32)
+	else:
+		kv_op = jnp.asarray(kv_lens).astype(jnp.int32).reshape((q.shape[0],))
+	return bias_op, seqlens, kv_op, bias_group
 
 
 def _seed_operand(dropout_seed):
 	"""The dropout seed as the 8-byte operand of the custom calls: uint32[2], low word first.
-	A Python int is split on the host; an array or tracer (the reference jits with a traced
-	dropout_seed, _flash_attention.py:91-92) is split with array operations, so nothing is
-	ever converted to a host scalar and one executable serves every seed."""
+	A Python int is split on the host (all 64 bits); an array or tracer (the reference jits with a traced
+	dropout_seed, _flash_attention.py:91-92) is split with array operations, so nothing is ever converted to a
+	host scalar and one executable serves every seed.  `flash_attention` / `flash_attention_call` convert the seed
+	BEFORE it reaches the differentiation rule: inside `jax.grad` a Python int argument would otherwise be traced
+	as a weakly typed int32 and a seed of 2^31 or more would overflow."""
 	if dropout_seed is None:
 		return jnp.zeros((2,), jnp.uint32)
 	if isinstance(dropout_seed, (int, np.integer)):
 		s = int(dropout_seed) & 0xFFFFFFFFFFFFFFFF
-		return jnp.array([s & 0xFFFFFFFF, s >> 32], dtype=jnp.uint32)
-	x = jnp.asarray(dropout_seed).reshape(())
+		return jnp.asarray(np.array([s & 0xFFFFFFFF, s >> 32], dtype=np.uint32))
+	x = jnp.asarray(dropout_seed)
+	if x.dtype == jnp.uint32 and x.shape == (2,):
+		return x  # already the operand
+	x = x.reshape(())
 	if x.dtype.itemsize == 8:
 		x = x.astype(jnp.uint64)
 		return jnp.stack([(x & 0xFFFFFFFF).astype(jnp.uint32), (x >> 32).astype(jnp.uint32)])
 	return jnp.stack([x.astype(jnp.uint32), jnp.zeros((), jnp.uint32)])
 
 
-def _fwd_scratch_bytes(q, k) -> int:
-	"""fa2_fwd_scratch_bytes for these shapes (host-only query; at least one aligned unit so the result is never empty)."""
-	import ctypes
-
+def _size_query(q, k, cfg: _Cfg, fn_names):
+	"""max over the named host-only size queries of the library for these shapes (at least one aligned unit so that
+	the result buffer is never empty)."""
 	from . import _lib
 
 	p = _lib.new_params()
 	p.B, p.Sq, p.Hq, p.D = (int(x) for x in q.shape)
 	p.Sk, p.Hkv = int(k.shape[1]), int(k.shape[2])
-	return max(int(_lib.load().fa2_fwd_scratch_bytes(ctypes.byref(p))), 256)
-
-
-def _bwd_scratch_bytes(q, k, causal=False) -> int:
-	"""Scratch of the backward for these shapes (host-only query): fa2_bwd_scratch_bytes, or the larger
-	fa2_bwd_split_scratch_bytes where the dK/dV kernel can split a key tile's work over workgroups."""
-	import ctypes
-
-	from . import _lib
-
-	p = _lib.new_params()
-	p.B, p.Sq, p.Hq, p.D = (int(x) for x in q.shape)
-	p.Sk, p.Hkv = int(k.shape[1]), int(k.shape[2])
-	p.causal = 1 if causal else 0  # (causal launches split further: their key tiles differ in length)
+	p.causal = 1 if cfg.causal else 0  # (causal backward launches split further: their key tiles differ in length)
+	p.has_window = 1 if cfg.has_window else 0
+	p.softcap = float(cfg.softcap)
 	lib = _lib.load()
-	return max(int(lib.fa2_bwd_scratch_bytes(ctypes.byref(p))), int(lib.fa2_bwd_split_scratch_bytes(ctypes.byref(p))), 256)
+	return max([int(getattr(lib, n)(ctypes.byref(p))) for n in fn_names] + [256])
 
 
-def _fwd_call(q, k, v, bias, seqlens, seed, attrs):
+def _fwd_call(ops: dict, cfg: _Cfg):
 	_register()
+	q, k = ops["q"], ops["k"]
 	B, Sq, Hq, _ = q.shape
-	out_types = (
-		jax.ShapeDtypeStruct(q.shape, q.dtype),
-		jax.ShapeDtypeStruct((B, Hq, Sq), jnp.float32),
-		jax.ShapeDtypeStruct((_fwd_scratch_bytes(q, k),), jnp.uint8),
+	out_types = dict(
+		o=jax.ShapeDtypeStruct(q.shape, q.dtype),
+		lse=jax.ShapeDtypeStruct((B, Hq, Sq), jnp.float32),
+		scratch=jax.ShapeDtypeStruct((_size_query(q, k, cfg, ("fa2_fwd_scratch_bytes",)),), jnp.uint8),
 	)
-	out, lse, _ = _ffi.ffi_call("fa2_fwd_ffi", out_types)(q, k, v, bias, seqlens, seed, **attrs)
-	return out, lse
+	res = _ffi_call("fa2_fwd_ffi", tuple(out_types[n] for n in spec.FWD_RESULTS))(*[ops[n] for n in spec.FWD_OPERANDS], **_attr_dict(cfg))
+	res = dict(zip(spec.FWD_RESULTS, res))
+	return res["o"], res["lse"]
 
 
-def _bwd_call(q, k, v, bias, seqlens, seed, out, lse, dout, attrs):
+def _bwd_call(ops: dict, cfg: _Cfg):
 	_register()
-	scratch_bytes = _bwd_scratch_bytes(q, k, attrs["causal"])
-	out_types = (
-		jax.ShapeDtypeStruct(q.shape, q.dtype),
-		jax.ShapeDtypeStruct(k.shape, k.dtype),
-		jax.ShapeDtypeStruct(v.shape, v.dtype),
-		jax.ShapeDtypeStruct((scratch_bytes,), jnp.uint8),
+	q, k, v = ops["q"], ops["k"], ops["v"]
+	B, Sq, Hq, _ = q.shape
+	Sk = k.shape[1]
+	scratch_bytes = _size_query(q, k, cfg, ("fa2_bwd_scratch_bytes", "fa2_bwd_split_scratch_bytes"))
+	out_types = dict(
+		dq=jax.ShapeDtypeStruct(q.shape, q.dtype),
+		dk=jax.ShapeDtypeStruct(k.shape, k.dtype),
+		dv=jax.ShapeDtypeStruct(v.shape, v.dtype),
+		# per-(batch, q-head) gradient of the additive term; 0 elements = not wanted
+		dbias=jax.ShapeDtypeStruct((B, Hq, Sq, Sk) if cfg.bias_grad else (0,), jnp.float32),
+		scratch=jax.ShapeDtypeStruct((scratch_bytes,), jnp.uint8),
 	)
-	dq, dk, dv, _ = _ffi.ffi_call("fa2_bwd_ffi", out_types)(q, k, v, bias, seqlens, seed, out, lse, dout, **attrs)
-	return dq, dk, dv
+	res = _ffi_call("fa2_bwd_ffi", tuple(out_types[n] for n in spec.BWD_RESULTS))(*[ops[n] for n in spec.BWD_OPERANDS], **_attr_dict(cfg))
+	res = dict(zip(spec.BWD_RESULTS, res))
+	return res["dq"], res["dk"], res["dv"], res["dbias"]
 
 
-# static: softmax_scale, dropout_prob, causal, varlen_mode (as in the reference, _flash_attention.py:119); dropout_seed
-# (argument 8) is an ordinary operand and may be traced
-@functools.partial(jax.custom_vjp, nondiff_argnums=(5, 6, 7, 9))
+# differentiable: q, k, v, bias; integer operands (seqlens, kv_lens, seed) get no cotangent; cfg is static
+@functools.partial(jax.custom_vjp, nondiff_argnums=(7,))
+def _attention(q, k, v, bias, seqlens, kv_lens, seed, cfg):
+	return _attention_fwd(q, k, v, bias, seqlens, kv_lens, seed, cfg)[0]
+
+
+def _attention_fwd(q, k, v, bias, seqlens, kv_lens, seed, cfg):
+	out, lse = _fwd_call(dict(q=q, k=k, v=v, bias=bias, seqlens=seqlens, kv_lens=kv_lens, seed=seed), cfg)
+	# residuals as in the reference (_flash_attention.py:64-66): q, k, v, bias, mask (here: lengths), out, lse, seed
+	return out, (q, k, v, bias, seqlens, kv_lens, seed, out, lse)
+
+
+def _attention_bwd(cfg, residual, dout):
+	q, k, v, bias, seqlens, kv_lens, seed, out, lse = residual
+	dq, dk, dv, dbias_full = _bwd_call(
+		dict(q=q, k=k, v=v, bias=bias, seqlens=seqlens, kv_lens=kv_lens, seed=seed, o=out, lse=lse, dout=dout), cfg)
+	dbias = None  # the reference returns no gradient for the bias (_flash_attention.py:88); `bias_grad=True` asks for one
+	if cfg.bias_grad:
+		dbias = _reduce_dbias(dbias_full, bias.shape, k.shape[2]).astype(bias.dtype)
+	return dq, dk, dv, dbias, None, None, None
+
+
+_attention.defvjp(_attention_fwd, _attention_bwd)
+
+
+def _reduce_dbias(full, bias_shape, Hkv):
+	"""[B, Hq, Sq, Sk] per-head gradient -> the shape of the bias: summed over the axes the kernels broadcast it on."""
+	B, Hq = full.shape[:2]
+	if bias_shape[1] == 1:
+		full = full.sum(axis=1, keepdims=True)
+	elif bias_shape[1] != Hq:
+		full = full.reshape(B, Hkv, Hq // Hkv, *full.shape[2:]).sum(axis=2)
+	if bias_shape[0] == 1 and B != 1:
+		full = full.sum(axis=0, keepdims=True)
+	return full
+
+
 def flash_attention_call(q, k, v, attention_mask=None, bias=None, softmax_scale=None, dropout_prob=0.0, causal=False,
-                         dropout_seed=None, varlen_mode=True):
-	return _fwd_rule(q, k, v, attention_mask, bias, softmax_scale, dropout_prob, causal, dropout_seed, varlen_mode)[0]
-
-
-def _fwd_rule(q, k, v, attention_mask, bias, softmax_scale, dropout_prob, causal, dropout_seed, varlen_mode):
-	bias_op, seqlens, bias_group = _prep(q, k, v, bias, attention_mask)
-	attrs = _attrs(q, softmax_scale, dropout_prob, causal, bias_group)
-	out, lse = _fwd_call(q, k, v, bias_op, seqlens, _seed_operand(dropout_seed), attrs)
-	return out, (q, k, v, bias, attention_mask, out, lse, dropout_seed)
-
-
-def _bwd_rule(softmax_scale, dropout_prob, causal, varlen_mode, residual, dout):
-	q, k, v, bias, attention_mask, out, lse, dropout_seed = residual
-	bias_op, seqlens, bias_group = _prep(q, k, v, bias, attention_mask)
-	attrs = _attrs(q, softmax_scale, dropout_prob, causal, bias_group)
-	dq, dk, dv = _bwd_call(q, k, v, bias_op, seqlens, _seed_operand(dropout_seed), out, lse, dout, attrs)
-	return dq, dk, dv, None, None, None  # no gradient for mask, bias, seed (_flash_attention.py:88)
-
-
-flash_attention_call.defvjp(_fwd_rule, _bwd_rule)
+                         dropout_seed=None, varlen_mode=True, *, kv_lens=None, window_size=None, softcap=0.0, bias_grad=False):
+	"""Argument list of the reference's `flash_attention_call` (_flash_attention.py:27-63) plus the keyword-only
+	operands the library has beyond it.  Head dim must be one the kernels are built for (`flash_attention` pads)."""
+	del varlen_mode  # padded batches are handled in-kernel from per-row lengths, never by packing
+	bias_op, seqlens, kv_op, bias_group = _operands(q, k, v, bias, attention_mask, kv_lens)
+	if bias_grad and (bias is None or not jnp.issubdtype(bias_op.dtype, jnp.floating)):
+		raise ValueError("bias_grad needs a floating-point bias")
+	if bias_grad and k.shape[1] % 4:
+		raise ValueError("bias_grad needs a key count that is a multiple of 4 (16-byte rows of the fp32 gradient)")
+	left, right = (-1, -1) if window_size is None else (int(window_size[0]), int(window_size[1]))
+	cfg = _Cfg(
+		scale=float(1.0 / math.sqrt(q.shape[-1]) if softmax_scale is None else softmax_scale),
+		dropout_p=float(dropout_prob),
+		causal=bool(causal),
+		bias_group=bool(bias_group),
+		has_window=window_size is not None,
+		window_left=left,
+		window_right=right,
+		softcap=float(softcap or 0.0),
+		bias_grad=bool(bias_grad),
+	)
+	return _attention(q, k, v, bias_op, seqlens, kv_op, _seed_operand(dropout_seed), cfg)
 
 
 def flash_attention(
@@ -195,14 +262,19 @@ def flash_attention(
 	causal: bool = False,
 	dropout_seed: tp.Optional[int] = None,
 	varlen_mode: bool = True,
+	*,
+	kv_lens=None,
+	window_size=None,
+	softcap: float = 0.0,
+	bias_grad: bool = False,
 ):
 	"""Same signature as the reference's `triton_flash_attention` (_flash_attention.py:125-157).
-	`dropout_seed` may be a Python int, an array or a tracer: it is an operand of the custom call.
-	A 4-D boolean mask becomes the bias where(mask, 0, finfo(dtype).min) (README.md:188)."""
-	if attention_mask is not None and attention_mask.ndim == 4:
-		assert bias is None, "Attention mask is not supported along with attention bias. Just use bias instead."
-		bias = jnp.where(attention_mask.astype(bool), jnp.zeros((), q.dtype), jnp.full((), jnp.finfo(q.dtype).min, q.dtype))
-		attention_mask = None
+	`dropout_seed` may be a Python int (all 64 bits are used), an array or a tracer: it is an operand of the custom call.
+	A 4-D boolean `attention_mask` is handed to the kernels as bytes (see `_operands`).  Keyword-only, not in the
+	reference: `kv_lens` int32 [B] (valid keys per batch row; may be combined with a bias and with Sq != Sk),
+	`window_size` = (left, right) (sliding window of refrence_call.py:55-75; a negative bound is none), `softcap`
+	(tanh soft-capping of refrence_call.py:48-51), `bias_grad` (also return the gradient of a floating-point bias;
+	costs an fp32 [B, Hq, Sq, Sk] intermediate)."""
 	# head dims other than 64 / 128 / 256: zero-pad to the next one (the reference pads to the next power of two,
 	# _forward_triton.py:525-526); pad and slice are differentiated by jax, the scale keeps the true head dim
 	D0 = q.shape[-1]
@@ -214,14 +286,15 @@ def flash_attention(
 			softmax_scale = 1.0 / math.sqrt(D0)
 		pad = ((0, 0), (0, 0), (0, 0), (0, D - D0))
 		q, k, v = jnp.pad(q, pad), jnp.pad(k, pad), jnp.pad(v, pad)
-	out = flash_attention_call(q, k, v, attention_mask, bias, softmax_scale, dropout_prob, causal, dropout_seed, varlen_mode)
+	out = flash_attention_call(q, k, v, attention_mask, bias, softmax_scale, dropout_prob, causal, dropout_seed, varlen_mode,
+	                           kv_lens=kv_lens, window_size=window_size, softcap=softcap, bias_grad=bias_grad)
 	return out if D == D0 else out[..., :D0]
 
 
 def dropout_mask(B, H, Sq, Sk, dropout_prob, dropout_seed):
 	_register()
 	out_type = jax.ShapeDtypeStruct((B, H, Sq, Sk), jnp.uint8)
-	return _ffi.ffi_call("fa2_dropout_mask_ffi", out_type)(_seed_operand(dropout_seed), dropout_p=np.float32(dropout_prob))
+	return _ffi_call("fa2_dropout_mask_ffi", out_type)(_seed_operand(dropout_seed), dropout_p=np.float32(dropout_prob))
 
 
 def place_on_least_used_gpu(query, key, value, bias):

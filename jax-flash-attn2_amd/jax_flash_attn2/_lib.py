@@ -80,7 +80,6 @@ EXPORTS = (
 	"fa2_fwd_scratch_bytes",
 	"fa2_dropout_mask",
 	"fa2_validate",
-	"fa2_bench_mfma",
 	"fa2_strerror",
 	"fa2_version",
 )
@@ -128,8 +127,6 @@ def load() -> ctypes.CDLL:
 		lib.fa2_dropout_mask.restype = ctypes.c_int
 		lib.fa2_validate.argtypes = [pp, ctypes.c_int]
 		lib.fa2_validate.restype = ctypes.c_int
-		lib.fa2_bench_mfma.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
-		lib.fa2_bench_mfma.restype = ctypes.c_int
 		lib.fa2_strerror.argtypes = [ctypes.c_int]
 		lib.fa2_strerror.restype = ctypes.c_char_p
 		lib.fa2_version.argtypes = []

@@ -76,6 +76,13 @@ def dropout_threshold(p_drop: float) -> int:
 	return min(int(math.floor(float(np.float32(p_drop)) * 65536.0)), 0xFFFF)
 
 
+def dropout_keep_scale(p_drop: float) -> float:
+	"""Factor applied to kept values: the reciprocal of the keep probability the 16-bit threshold really gives,
+	65536 / (65536 - threshold) - the reference's 1 / (1 - p) (_forward_triton.py:435-438) for the p that the
+	threshold realises, so that E[O] equals the output without dropout exactly."""
+	return 65536.0 / (65536.0 - dropout_threshold(p_drop))
+
+
 def dropout_keep_mask(seed: int, p_drop: float, B: int, H: int, Sq: int, Sk: int, pos_offset=(0, 0, 0)) -> np.ndarray:
 	"""keep[b,h,i,j] (bool).  `pos_offset` = (b0, h0, i0) shifts the batch / head /
 	row indices, for checking a slice of a larger problem (i0 must be even).
@@ -231,7 +238,7 @@ def attention_fwd(q, k, v, bias=None, causal=False, scale=None, seqlens=None,
 	pd = p
 	if p_drop > 0.0:
 		keep = dropout_keep_mask(seed, p_drop, B, Hq, Sq, Sk, pos_offset)
-		pd = np.where(keep, p, 0.0) / dtype(1.0 - float(np.float32(p_drop)))
+		pd = np.where(keep, p, 0.0) * dtype(dropout_keep_scale(p_drop))
 	vf = np.repeat(np.asarray(v, dtype=dtype), r, axis=2)
 	o = _pv(pd, vf)
 	if return_probs:
@@ -263,7 +270,7 @@ def attention_bwd(q, k, v, dO, bias=None, causal=False, scale=None, seqlens=None
 	dpd = _qk(dOf, vf)
 	if p_drop > 0.0:
 		keep = dropout_keep_mask(seed, p_drop, B, Hq, Sq, Sk, pos_offset)
-		dp = np.where(keep, dpd, 0.0) / dtype(1.0 - float(np.float32(p_drop)))
+		dp = np.where(keep, dpd, 0.0) * dtype(dropout_keep_scale(p_drop))
 	else:
 		dp = dpd
 	if o_stored is not None:

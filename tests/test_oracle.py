@@ -55,6 +55,20 @@ def test_dropout_mask_definition_and_rate():
 	assert O.dropout_keep_mask(1, 0.0, 1, 1, 8, 8).all()
 
 
+@pytest.mark.parametrize("p", [0.0, 1e-6, 0.1, 0.25, 0.3, 0.5, 0.999, 0.99999])
+def test_dropout_keep_scale_makes_the_expectation_exact(p):
+	"""Kept values are scaled by the reciprocal of the keep probability the 16-bit threshold really gives: over the
+	65536 equally likely values of an element, sum(keep) * scale is exactly the number of values - so E[O] is the
+	output without dropout for every p, also where p is not a multiple of 2^-16 and below 2^-16 (nothing dropped,
+	nothing rescaled).  The reference's factor 1 / (1 - p) (_forward_triton.py:435-438) is the same number for the
+	probability that is realised."""
+	thr = O.dropout_threshold(p)
+	kept = int((np.arange(65536) >= thr).sum())
+	assert kept >= 1
+	assert kept * O.dropout_keep_scale(p) == pytest.approx(65536.0, rel=1e-15)
+	assert abs(O.dropout_keep_scale(p) - 1.0 / (1.0 - float(np.float32(p)))) <= 2.0 ** -16 * O.dropout_keep_scale(p) ** 2 * 1.0001 or thr == 0xFFFF
+
+
 def _rand(rng, B, Sq, Sk, Hq, Hkv, D):
 	return (rng.normal(size=(B, Sq, Hq, D)), rng.normal(size=(B, Sk, Hkv, D)), rng.normal(size=(B, Sk, Hkv, D)),
 	        rng.normal(size=(B, Sq, Hq, D)))
@@ -228,6 +242,32 @@ def test_key_lengths_equal_an_explicit_key_mask():
 	# a length of zero: no key at all
 	o, lse = O.attention_fwd(q, k, v, kv_lens=[0, 14])
 	assert np.all(o[0] == 0) and np.all(np.isneginf(lse[0])) and np.all(np.isfinite(lse[1]))
+
+
+def test_key_lengths_keep_the_window_aligned_to_the_full_key_count():
+	"""Chosen semantics, on purpose different from the reference's naive attention: there a key_padding_mask moves the
+	window (row i is aligned with key i + valid_keys - Sq, refrence_call.py:58-66); `kv_lens` is padding at the end of
+	a key axis whose positions keep their meaning, so row i stays aligned with key i + Sk - Sq and the length only
+	removes keys.  Written out for Sq 3, Sk 8, window (1, 1), kv_len 6."""
+	got = O.allowed_mask(1, 3, 8, False, kv_lens=[6], window=(1, 1))[0].astype(int)
+	expect = np.array([
+		# keys 0 1 2 3 4 5 | 6 7 (padding)
+		[0, 0, 0, 0, 1, 1, 0, 0],  # row 0 <-> key 5: keys 4..6, key 6 is padding
+		[0, 0, 0, 0, 0, 1, 0, 0],  # row 1 <-> key 6: keys 5..7, only 5 is valid
+		[0, 0, 0, 0, 0, 0, 0, 0],  # row 2 <-> key 7: keys 6..7, none valid -> O = 0, lse = -inf
+	])
+	assert np.array_equal(got, expect)
+	# the reference's alignment (to the valid length: row i <-> key i + 6 - 3) would have given another set of keys
+	ref_style = O.allowed_mask(1, 3, 6, False, window=(1, 1))[0].astype(int)
+	assert not np.array_equal(got[:, :6], ref_style)
+	# same with the causal flag: row i sees keys <= i + Sk - Sq that are valid
+	got = O.allowed_mask(1, 3, 8, True, kv_lens=[6])[0]
+	assert np.array_equal(got, (np.arange(8)[None, :] <= np.arange(3)[:, None] + 5) & (np.arange(8)[None, :] < 6))
+	rng = np.random.default_rng(3)
+	q, k, v = rng.normal(size=(1, 3, 2, 4)), rng.normal(size=(1, 8, 2, 4)), rng.normal(size=(1, 8, 2, 4))
+	o, lse = O.attention_fwd(q, k, v, kv_lens=[6], window=(1, 1))
+	assert np.all(o[0, 2] == 0) and np.all(np.isneginf(lse[0, :, 2]))
+	assert np.allclose(o[0, 1], v[0, 5])  # a single key: its value
 
 
 def test_sliding_window_is_the_local_mask_of_the_naive_reference():

@@ -447,6 +447,18 @@ def test_sliding_window(window):
 	g_ref = O.attention_bwd(f64(q), f64(k), f64(v), f64(do), kv_lens=[150, 90], window=window)
 	assert np.abs(out.detach().float().cpu().numpy() - o_ref).max() <= TOL_O[torch.bfloat16]
 	check_grads((qq.grad,), (g_ref[0],), f"window {window} with key lengths")
+	# cross lengths with key lengths: the window (and the causal flag) stay aligned to the FULL key count, row i <-> key
+	# i + Sk - Sq, the length only removes keys (the oracle's test_key_lengths_keep_the_window_aligned_... spells it out)
+	for causal in (False, True):
+		q, k, v, do, _ = make_inputs(2, 130, 300, 4, 2, 128, torch.bfloat16, 53)
+		kw = dict(causal=causal, kv_lens=[300, 201], window=window)
+		o_ref, lse_ref = O.attention_fwd(f64(q), f64(k), f64(v), **kw)
+		g_ref = O.attention_bwd(f64(q), f64(k), f64(v), f64(do), **kw)
+		kl = torch.tensor([300, 201], dtype=torch.int32, device=DEV)
+		o, lse = op.fwd(_dev(q), _dev(k), _dev(v), None, None, None, 0.0, causal, 0, kl, window)
+		gr = op.bwd(_dev(q), _dev(k), _dev(v), o, lse, _dev(do), None, None, None, 0.0, causal, 0, kl, window)
+		check_forward(o, lse, o_ref, lse_ref, torch.bfloat16, f"window {window} Sq130 Sk300 kv_lens causal={causal}")
+		check_grads(gr, g_ref, f"window {window} Sq130 Sk300 kv_lens causal={causal}")
 
 
 @pytest.mark.parametrize("cap", [1.0, 5.0, 30.0])
@@ -518,8 +530,9 @@ def test_mask_as_finfo_min_bias():
 )
 @pytest.mark.parametrize("D,dtype", [(64, torch.bfloat16), (128, torch.float16), (256, torch.bfloat16)])
 def test_bias_gradient(bshape, D, dtype):
-	"""fa2_params.dbias (the dQ kernel writes the per-head gradient of the additive term, the operator sums it over the
-	axes the bias is broadcast on) against the oracle; ragged tiles, causal, dropout, key lengths; dq / dk / dv unchanged."""
+	"""fa2_params.dbias in the shape of the bias (the dQ kernel adds the per-head gradient of the additive term into it,
+	with atomic adds on the axes the bias is broadcast on) against the oracle; ragged tiles, causal, dropout, key lengths;
+	dq / dk / dv unchanged."""
 	B, Sq, Sk, Hq, Hkv = 2, 160, 203, 4, 2
 	for causal, p, kv_lens in ((False, 0.0, None), (True, 0.2, None), (False, 0.0, [150, 64])):
 		q, k, v, do, bias = make_inputs(B, Sq, Sk, Hq, Hkv, D, dtype, 5, (*bshape, Sq, Sk))
@@ -541,13 +554,14 @@ def test_bias_gradient(bshape, D, dtype):
 
 
 def test_bias_gradient_through_autograd_and_softcap():
-	"""A bias that requires a gradient gets one from the operator's differentiation rule (the reference returns None for
-	it, _flash_attention.py:88); with soft-capping the bias gradient does not carry the 1 - tanh^2 factor."""
+	"""A bias that requires a gradient gets one from the operator's differentiation rule when the caller asks for it with
+	`bias_grad=True` (the reference returns None for it, _flash_attention.py:88, and so does this operator by default); with
+	soft-capping the bias gradient does not carry the 1 - tanh^2 factor."""
 	B, Sq, Sk, Hq, Hkv, D = 1, 96, 130, 4, 4, 64
 	q, k, v, do, bias = make_inputs(B, Sq, Sk, Hq, Hkv, D, torch.bfloat16, 2, (1, 1, Sq, Sk), bias_dtype=torch.float32)
 	ref = O.attention_bwd(f64(q), f64(k), f64(v), f64(do), f64(bias), causal=True, softcap=2.0, return_dbias=True)
 	qd, kd, vd, bd = (_dev(t).requires_grad_(True) for t in (q, k, v, bias))
-	out = op.flash_attention(qd, kd, vd, bias=bd, causal=True, softcap=2.0)
+	out = op.flash_attention(qd, kd, vd, bias=bd, causal=True, softcap=2.0, bias_grad=True)
 	out.backward(_dev(do))
 	torch.cuda.synchronize()
 	check_grads((qd.grad, kd.grad, vd.grad), ref[:3], "autograd with bias gradient")
@@ -558,6 +572,10 @@ def test_bias_gradient_through_autograd_and_softcap():
 	b2 = _dev(bias)
 	op.flash_attention(qd2, _dev(k), _dev(v), bias=b2, causal=True, softcap=2.0).backward(_dev(do))
 	assert b2.grad is None and torch.equal(qd2.grad, qd.grad)
+	# ... nor for a bias that requires one but was not asked for (as in the reference)
+	qd3, b3 = _dev(q).requires_grad_(True), _dev(bias).requires_grad_(True)
+	op.flash_attention(qd3, _dev(k), _dev(v), bias=b3, causal=True, softcap=2.0).backward(_dev(do))
+	assert b3.grad is None and torch.equal(qd3.grad, qd.grad)
 
 
 @pytest.mark.parametrize("causal", [False, True])
@@ -675,7 +693,7 @@ def test_kernels_apply_exactly_the_exported_mask():
 	zero = torch.zeros(B, S, H, D, dtype=dtype, device=DEV)
 	ones = torch.ones(B, S, H, D, dtype=dtype, device=DEV)
 	keep = O.dropout_keep_mask(seed, p, B, H, S, S)  # [B,H,i,j]
-	inv = 1.0 / (1.0 - float(np.float32(p)))
+	inv = O.dropout_keep_scale(p)
 	# forward: O[b,i,h,j] = keep[b,h,i,j] / (S (1-p))
 	o, lse = op.fwd(zero, eye, eye, None, None, None, p, False, seed)
 	got = (o.float().permute(0, 2, 1, 3).cpu().numpy() * S / inv) > 0.5
