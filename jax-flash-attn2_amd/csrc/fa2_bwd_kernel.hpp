@@ -214,12 +214,10 @@ FA2_DEV void bwd_dkdv_tile(const KArgs& a, const int nt, const int hk, const int
 	doload.init(a.dout.ss, tid);
 	TileLoader<128, BMQ, NT> bload;
 	if constexpr (BIAS_LDS) bload.init(a.bias_sm, tid);
-	// Streamed tile `step`: head by head, and for each head the query tiles from this workgroup's first
-	// one up.  (Measured alternative: all key tiles of a (batch, kv-head) walking the query tiles in
-	// the same order at the same time, so that each Q / dO tile is fetched from HBM once per XCD -
-	// the kernel gets 4 - 6 % slower on the 4096-token workload and no faster on the 32768-token
-	// one: it is not bound by that traffic, and 32 workgroups asking for the same lines at the same
-	// moment wait on each other.)
+	// Streamed tile `step` in the order `order` asks for (see above).  Head by head is what a workgroup with one key
+	// tile does: walking the query tiles outermost there measured 2 - 3 % slower (the workgroups of a KV group differ in
+	// length and drift apart either way).  The two query-tile-outermost orders belong to the paired tiles of
+	// bwd_dkdv_kernel, where all workgroups are equally long and stay together.
 	auto decode_step = [&](int step, int& hq, int& m0) __attribute__((always_inline)) {
 		int hi, i;
 		if (order == 0) {
@@ -231,33 +229,42 @@ FA2_DEV void bwd_dkdv_tile(const KArgs& a, const int nt, const int hk, const int
 			hi = hi >= r ? hi - r : hi;
 			i = order == 2 ? nq - 1 - t : t;
 		}
-		hq = hk * r + hi;
-		m0 = (q_lo + i) * BMQ;
+		// (explicitly scalar: the results feed address arithmetic in branches that only some lanes take, and values the
+		// compiler has to merge across such a branch end up in vector registers - every multiply of the tile's base
+		// address then runs on the vector ALU)
+		hq = __builtin_amdgcn_readfirstlane(hk * r + hi);
+		m0 = __builtin_amdgcn_readfirstlane((q_lo + i) * BMQ);
 	};
 	// start the copies of streamed tile `step` (rows beyond Sq are fetched from the last valid row)
-	auto issue_tile = [&](int step, FA2_LDS char* qdst, FA2_LDS char* dodst) __attribute__((always_inline)) {
-		int hq, m0;
-		decode_step(step, hq, m0);
-		int rows = a.Sq - m0 < BMQ ? a.Sq - m0 : BMQ;
-		const char* qb_ = a.q.ptr + (int64_t)b * a.q.sb + (int64_t)hq * a.q.sh + (int64_t)m0 * a.q.ss;
-		const char* db_ = a.dout.ptr + (int64_t)b * a.dout.sb + (int64_t)hq * a.dout.sh + (int64_t)m0 * a.dout.ss;
-		qload.load(qdst, qb_, a.q.ss, rows, tid);
-		doload.load(dodst, db_, a.dout.ss, rows, tid);
+	// base addresses of a streamed tile, as explicitly scalar values (computed in uniform control flow, ahead of the
+	// branch in which some lanes fetch the statistics)
+	struct TileBase {
+		const char *q, *dout, *bias;
+	};
+	auto tile_base = [&](int hq, int m0) __attribute__((always_inline)) {
+		TileBase t;
+		t.q = TileLoader<D, BMQ, NT>::uniform(a.q.ptr + (int64_t)b * a.q.sb + (int64_t)hq * a.q.sh + (int64_t)m0 * a.q.ss);
+		t.dout = TileLoader<D, BMQ, NT>::uniform(a.dout.ptr + (int64_t)b * a.dout.sb + (int64_t)hq * a.dout.sh + (int64_t)m0 * a.dout.ss);
+		t.bias = nullptr;
 		if constexpr (BIAS_LDS) {
 			int hb = a.bias_group ? hk : hq;
-			const char* bb_ = a.bias + (int64_t)b * a.bias_sb + (int64_t)hb * a.bias_sh + (int64_t)m0 * a.bias_sm + (int64_t)n0 * 2;
-			bload.load(lds_bias + ((step - s_lo) & 1) * BIAS_BYTES, bb_, a.bias_sm, rows, tid, (a.Sk - n0) >> 3);
+			t.bias = TileLoader<D, BMQ, NT>::uniform(a.bias + (int64_t)b * a.bias_sb + (int64_t)hb * a.bias_sh + (int64_t)m0 * a.bias_sm + (int64_t)n0 * 2);
 		}
+		return t;
+	};
+	auto issue_tile = [&](int step, const TileBase& tb, int m0, FA2_LDS char* qdst, FA2_LDS char* dodst) __attribute__((always_inline)) {
+		int rows = a.Sq - m0 < BMQ ? a.Sq - m0 : BMQ;
+		qload.load(qdst, tb.q, a.q.ss, rows, tid);
+		doload.load(dodst, tb.dout, a.dout.ss, rows, tid);
+		if constexpr (BIAS_LDS) bload.load(lds_bias + ((step - s_lo) & 1) * BIAS_BYTES, tb.bias, a.bias_sm, rows, tid, (a.Sk - n0) >> 3);
 	};
 	// per-row statistics of a tile: thread t < BMQ fetches lse, t in [BMQ, 2 BMQ) fetches delta.
 	// The value is only touched again in store_stat(), a whole step later: nothing here may wait for the load.
 	const int stat_row = tid % BMQ;
 	const float* stat_src = tid < BMQ ? a.lse : a.delta;
-	auto fetch_stat = [&](int step) -> float {
+	auto fetch_stat = [&](int hq, int m0) -> float {
 		float x = 0.f;
 		if (tid < 2 * BMQ) {
-			int hq, m0;
-			decode_step(step, hq, m0);
 			int i = m0 + stat_row;
 			i = i < a.Sq ? i : a.Sq - 1;
 			x = stat_src[((int64_t)b * a.Hq + hq) * a.Sq + i];
@@ -721,9 +728,12 @@ FA2_DEV void bwd_dkdv_tile(const KArgs& a, const int nt, const int hk, const int
 		static_assert(QB <= 4, "");
 	};
 
+	// (q-head, first row) of the streamed tile the next step computes on: decoded once, when its copies are started
+	int cur_hq = 0, cur_m0 = 0;
 	if (s_hi > s_lo) {
-		issue_tile(s_lo, lds, lds + TILE_BYTES);
-		store_stat(fetch_stat(s_lo), 0);
+		decode_step(s_lo, cur_hq, cur_m0);
+		issue_tile(s_lo, tile_base(cur_hq, cur_m0), cur_m0, lds, lds + TILE_BYTES);
+		store_stat(fetch_stat(cur_hq, cur_m0), 0);
 	}
 
 	// One pipeline step: publish streamed tile `step`, start the copies of the next, compute.
@@ -732,16 +742,18 @@ FA2_DEV void bwd_dkdv_tile(const KArgs& a, const int nt, const int hk, const int
 		wait_async_loads();
 		__syncthreads();
 		float next_stat = 0.f;
+		int nxt_hq = 0, nxt_m0 = 0;
 		const bool has_next = step + 1 < s_hi;
 		if (has_next) {
 			// statistics first: loads return in order, so waiting for this small load later
 			// does not wait for the tile copies issued after it
-			next_stat = fetch_stat(step + 1);
-			issue_tile(step + 1, lds + (buf ^ 1) * (2 * TILE_BYTES), lds + (buf ^ 1) * (2 * TILE_BYTES) + TILE_BYTES);
+			decode_step(step + 1, nxt_hq, nxt_m0);
+			const TileBase tb = tile_base(nxt_hq, nxt_m0);
+			next_stat = fetch_stat(nxt_hq, nxt_m0);
+			issue_tile(step + 1, tb, nxt_m0, lds + (buf ^ 1) * (2 * TILE_BYTES), lds + (buf ^ 1) * (2 * TILE_BYTES) + TILE_BYTES);
 		}
 		{
-			int hq, m0;
-			decode_step(step, hq, m0);
+			const int hq = cur_hq, m0 = cur_m0;
 			bool skip = false;
 			if constexpr (decltype(masked_tag)::value) {
 				// wave-uniform: nothing to do for (rows m0.., keys wn0..)?
@@ -764,6 +776,8 @@ FA2_DEV void bwd_dkdv_tile(const KArgs& a, const int nt, const int hk, const int
 			boffq[1] ^= BIAS_BYTES;
 		}
 		if (has_next) store_stat(next_stat, buf ^ 1);
+		cur_hq = nxt_hq;
+		cur_m0 = nxt_m0;
 		// The load of the statistics has completed on every path out of the step.  Without this use the compiler
 		// takes the load for possibly still in flight at the top of the next step (it cannot tell that the two
 		// `has_next` tests agree) and guards the first reuse of its register there with s_waitcnt vmcnt(0) - which
