@@ -66,9 +66,64 @@ __global__ __launch_bounds__(256) void bwd_delta_kernel(const KArgs a) {
 //   2  the same with the query tiles descending.
 // With 1 and 2 every workgroup of a KV group that walks in the same direction is at the same query tile at the same
 // time, whatever its key tile - the tiles of Q / dO they stream are then fetched from memory once per XCD.
-template <typename T, int D, int NW, int QB, bool BIAS, bool DROP, bool BIAS_T, bool CAP>
-FA2_DEV void bwd_dkdv_tile(const KArgs& a, const int nt, const int hk, const int b, const int hsi, const int hsplit, const int order,
-                           const int rot) {
+// What depends on the batch row only: valid rows / keys and the causal alignment, the dropout key.
+struct DkdvRow {
+	int sq_eff, sk_eff, off;
+	uint32_t drop_k0, drop_k1;
+};
+
+template <bool DROP>
+FA2_DEV DkdvRow dkdv_row(const KArgs& a, int b) {
+	DkdvRow rw;
+	rw.sq_eff = a.Sq;
+	rw.sk_eff = a.Sk;
+	if (a.seqlens) {
+		int len = a.seqlens[b];
+		len = len < 0 ? 0 : (len > a.Sk ? a.Sk : len);
+		rw.sq_eff = len < a.Sq ? len : a.Sq;
+		rw.sk_eff = len;
+	}
+	rw.off = rw.sk_eff - rw.sq_eff;
+	if (a.kv_lens) {  // key padding only: the causal alignment keeps counting from the full key count
+		int len = a.kv_lens[b];
+		len = len < 0 ? 0 : len;
+		rw.sk_eff = len < rw.sk_eff ? len : rw.sk_eff;
+	}
+	// dropout key: from the parameter block, or from device memory when the caller keeps it there
+	rw.drop_k0 = a.drop_k0;
+	rw.drop_k1 = a.drop_k1;
+	if constexpr (DROP) {
+		if (a.seed_dev) {
+			rw.drop_k0 = a.seed_dev[0];
+			rw.drop_k1 = a.seed_dev[1];
+		}
+	}
+	return rw;
+}
+
+// K, V rows of this lane's key of key tile nt as B operands: the lane holds X[key][16 ks + 8 g .. + 7].
+template <typename T, int D, int NW>
+FA2_DEV void dkdv_load_kv(const KArgs& a, int nt, int hk, int b, typename T::V8 (&kf)[D / 16], typename T::V8 (&vf)[D / 16]) {
+	typedef typename T::V8 V8;
+	const int tid = threadIdx.x, lane = tid & 63;
+	const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+	const int g = lane >> 5, c = lane & 31;
+	const int jcol = nt * (NW * 32) + 32 * w + c;
+	int j = jcol < a.Sk ? jcol : a.Sk - 1;
+	const char* kp = a.k.ptr + (int64_t)b * a.k.sb + (int64_t)hk * a.k.sh + (int64_t)j * a.k.ss + g * 16;
+	const char* vp = a.v.ptr + (int64_t)b * a.v.sb + (int64_t)hk * a.v.sh + (int64_t)j * a.v.ss + g * 16;
+#pragma unroll
+	for (int ks = 0; ks < D / 16; ++ks) {
+		kf[ks] = *(const V8*)(kp + ks * 32);
+		vf[ks] = *(const V8*)(vp + ks * 32);
+	}
+}
+
+// WALKS: `order` is a run-time value (the paired kernel); otherwise the tile is walked head by head and `order_rt` is not looked at.
+template <typename T, int D, int NW, int QB, bool BIAS, bool DROP, bool BIAS_T, bool CAP, bool WALKS>
+FA2_DEV void bwd_dkdv_tile(const KArgs& a, const int nt, const int hk, const int b, const int hsi, const int hsplit, const int order_rt,
+                           const int rot, const DkdvRow& rw) {
+	const int order = WALKS ? order_rt : 0;
 	static_assert(!CAP || (BIAS && !BIAS_T), "soft-capping runs on the plain path with bias");
 	typedef typename T::V8 V8;
 	constexpr int BN = NW * 32;     // keys per workgroup
@@ -116,50 +171,16 @@ FA2_DEV void bwd_dkdv_tile(const KArgs& a, const int nt, const int hk, const int
 	// "nothing to do for this wave") then stays in scalar registers and scalar branches
 	const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int g = lane >> 5, c = lane & 31;
-	// dropout key: from the parameter block, or from device memory when the caller keeps it there
-	uint32_t drop_k0 = a.drop_k0, drop_k1 = a.drop_k1;
-	if constexpr (DROP) {
-		if (a.seed_dev) {
-			drop_k0 = a.seed_dev[0];
-			drop_k1 = a.seed_dev[1];
-		}
-	}
-
-	// (a workgroup may handle two key tiles one after the other: the LDS buffers of the previous one are free
-	// once every wave has left its last step)
-	__syncthreads();
+	const uint32_t drop_k0 = rw.drop_k0, drop_k1 = rw.drop_k1;
 	const int r = a.Hq / a.Hkv;
-
-	int sq_eff = a.Sq, sk_eff = a.Sk;
-	if (a.seqlens) {
-		int len = a.seqlens[b];
-		len = len < 0 ? 0 : (len > a.Sk ? a.Sk : len);
-		sq_eff = len < a.Sq ? len : a.Sq;
-		sk_eff = len;
-	}
-	const int off = sk_eff - sq_eff;
-	if (a.kv_lens) {  // key padding only: the causal alignment keeps counting from the full key count
-		int len = a.kv_lens[b];
-		len = len < 0 ? 0 : len;
-		sk_eff = len < sk_eff ? len : sk_eff;
-	}
+	const int sq_eff = rw.sq_eff, sk_eff = rw.sk_eff, off = rw.off;
 	const int n0 = nt * BN;
 	const int wn0 = n0 + 32 * w;
 	const int jcol = wn0 + c;  // this lane's key
 
 	// K, V rows of this lane's key as B operands: lane holds X[jcol][16ks + 8g .. +7]
 	V8 kf[KS], vf[KS];
-	{
-		int j = jcol < a.Sk ? jcol : a.Sk - 1;
-		const char* kp = a.k.ptr + (int64_t)b * a.k.sb + (int64_t)hk * a.k.sh + (int64_t)j * a.k.ss + g * 16;
-		const char* vp = a.v.ptr + (int64_t)b * a.v.sb + (int64_t)hk * a.v.sh + (int64_t)j * a.v.ss + g * 16;
-#pragma unroll
-		for (int ks = 0; ks < KS; ++ks) {
-			kf[ks] = *(const V8*)(kp + ks * 32);
-			vf[ks] = *(const V8*)(vp + ks * 32);
-		}
-	}
-
+	dkdv_load_kv<T, D, NW>(a, nt, hk, b, kf, vf);
 	// The fragments must have arrived before the loop over streamed tiles starts.  Otherwise the compiler places its
 	// waits for these loads (s_waitcnt vmcnt) at their first uses inside the loop - it does not see the wait that
 	// publishes a tile - where the same counter also counts the tile copies in flight: every step would then wait
@@ -172,6 +193,7 @@ FA2_DEV void bwd_dkdv_tile(const KArgs& a, const int nt, const int hk, const int
 		else
 			asm volatile("; K / V fragment present" : "+v"(kf[ks]), "+v"(vf[ks]));
 	}
+
 
 	f32x16 dk[DB], dv[DB];
 #pragma unroll
@@ -864,7 +886,9 @@ FA2_DEV void bwd_dkdv_tile(const KArgs& a, const int nt, const int hk, const int
 // blockIdx.x -> (key tile or pair of key tiles, kv head, batch); the key tiles of one (b, kv head) stay on one XCD.
 // BIAS_T: the bias has the element type of q / k / v (no run-time type dispatch per value)
 // CAP: tanh soft-capping of the scores (see the forward kernel); the bias itself may then be absent
-template <typename T, int D, int NW, int QB, bool BIAS, bool DROP, bool BIAS_T, bool CAP = false>
+// PAIR: the instantiation for launches that give a workgroup two key tiles (a.kv_pair); the launcher picks it only then,
+// so that every other launch runs the kernel with the one walk as a compile-time constant.
+template <typename T, int D, int NW, int QB, bool BIAS, bool DROP, bool BIAS_T, bool CAP = false, bool PAIR = false>
 __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 	// (with the steps of a key tile split over workgroups: the parts of one key tile are adjacent)
 	int hk, b, within;
@@ -901,28 +925,28 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(const KArgs a) {
 		hk = grp % a.Hkv;
 		b = grp / a.Hkv;
 	}
-	const int r = a.Hq / a.Hkv;
-	// (head dim 256 sits at the edge of the register file: it keeps the one walk, as a compile-time constant)
-	constexpr bool WALKS = D <= 128;
-	if constexpr (!WALKS) {
-		bwd_dkdv_tile<T, D, NW, QB, BIAS, DROP, BIAS_T, CAP>(a, within, hk, b, hsi, hsplit, 0, 0);
-	} else if (a.kv_pair) {
+	const DkdvRow rw = dkdv_row<DROP>(a, b);
+	if constexpr (!PAIR) {
+		// one key tile, head by head (early key tiles see the most query rows under a causal mask: first)
+		bwd_dkdv_tile<T, D, NW, QB, BIAS, DROP, BIAS_T, CAP, false>(a, within, hk, b, hsi, hsplit, 0, 0, rw);
+	} else {
 		// Causal self-attention: key tile p streams every query tile from p up, so a workgroup takes tile p and tile
 		// ntiles - 1 - p one after the other - every workgroup then has the same number of steps (no CU waits for the
 		// longest tile, no gaps in the dispatch), and the two walks are arranged so that all workgroups of a KV group
 		// stay together: the long tile runs from the last query tile DOWN (all workgroups start at the same tile and
-		// drop out one by one), the short tile from its diagonal UP (a workgroup that has finished tile p, one step
-		// later than the workgroup of p + 1, joins that workgroup's second walk exactly where it is now).  At any
+		// drop out one by one), the short tile from its diagonal UP (a workgroup that has finished tile p, one query
+		// tile later than the workgroup of p + 1, joins that workgroup's second walk exactly where it is now).  At any
 		// time the KV group reads two fronts of Q / dO tiles, not one per workgroup.
-		const int ntiles = a.kv_ntiles;
-		const int rot = within % r;
+		const int r = a.Hq / a.Hkv;
+		const int partner = a.kv_ntiles - 1 - within;
 		// (an odd number of tiles: the middle one is its own partner)
-		const int npass = ntiles - 1 - within == within ? 1 : 2;
-		for (int pass = 0; pass < npass; ++pass)
-			bwd_dkdv_tile<T, D, NW, QB, BIAS, DROP, BIAS_T, CAP>(a, pass == 0 ? within : ntiles - 1 - within, hk, b, 0, 1, pass == 0 ? 2 : 1, rot);
-	} else {
-		// early key tiles see the most query rows under a causal mask: first
-		bwd_dkdv_tile<T, D, NW, QB, BIAS, DROP, BIAS_T, CAP>(a, within, hk, b, hsi, hsplit, a.kv_order, a.kv_order ? within % r : 0);
+		const int npass = partner != within ? 2 : 1;
+		const int rot = within % r;
+		for (int pass = 0; pass < npass; ++pass) {
+			bwd_dkdv_tile<T, D, NW, QB, BIAS, DROP, BIAS_T, CAP, true>(a, pass == 0 ? within : partner, hk, b, 0, 1, 2 - pass, rot, rw);
+			// (the LDS buffers of the first tile are free once every wave has left its last step)
+			if (pass + 1 < npass) __syncthreads();
+		}
 	}
 }
 
@@ -1601,12 +1625,12 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 		// ntiles - 1 - p one after the other (see bwd_dkdv_kernel).  Measured on the 4096-token workload (B4 Hq32 Hkv8):
 		// dK/dV kernel 1.032 -> 1.000 ms and 1318 -> 437 MiB fetched from memory (324 MiB of operands); on the
 		// 32768-token one 31.7 -> 30.3 ms and 87 -> 4.8 GiB (1.14 GiB of operands).  Walking the query tiles outermost
-		// WITHOUT the pairing (kv_order 1 / 2 on one tile per workgroup) measured slower than head by head: 1.065 /
+		// WITHOUT the pairing (one tile per workgroup, ascending or descending) measured slower than head by head: 1.065 /
 		// 1.051 ms, so everything else keeps that order.
-		a.kv_order = 0;
 		a.kv_pair = 0;
 		a.kv_ntiles = a.mtiles;
-		if (D <= 128 && hs == 1 && a.causal && a.win_left < 0 && a.Sq == a.Sk && !a.seqlens && !a.kv_lens && a.xcd_remap <= 1 && a.mtiles >= 2) {
+		// (from 16 key tiles on: B16 H16 S1000, 8 tiles of one q-head each, measured 0.218 ms one tile per workgroup and 0.224 ms paired)
+		if (D <= 128 && !BIAS && hs == 1 && a.causal && a.win_left < 0 && a.Sq == a.Sk && !a.seqlens && !a.kv_lens && a.xcd_remap <= 1 && a.mtiles >= 16) {
 			const int64_t pairs = (int64_t)((a.mtiles + 1) / 2) * groups;
 			if (pairs % kNumCU == 0 || pairs >= 8 * kNumCU) {
 				a.kv_pair = 1;
@@ -1624,7 +1648,10 @@ hipError_t launch_bwd_v(KArgs& a, hipStream_t s) {
 			hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, C::KV_NW, QBV, BIAS, DROP, false, BIAS>), grid, block, 0, s, a);
 		else if (typed)
 			hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, C::KV_NW, QBV, BIAS, DROP, BIAS>), grid, block, 0, s, a);
-		else
+		else if (a.kv_pair) {
+			// (only instantiated where the launcher can choose it: no bias, head dim up to 128)
+			if constexpr (D <= 128 && !BIAS) hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, C::KV_NW, QBV, BIAS, DROP, false, false, true>), grid, block, 0, s, a);
+		} else
 			hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, C::KV_NW, QBV, BIAS, DROP, false>), grid, block, 0, s, a);
 		if (hs > 1) {
 			int64_t total = (int64_t)a.B * a.Hkv * a.Sk * 2 * (D / 8);

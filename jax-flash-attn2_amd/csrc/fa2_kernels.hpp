@@ -46,10 +46,9 @@ struct KArgs {
 	// kernel sums, scales and stores them.  1 = no split.
 	int kv_hsplit;
 	float* dkv_part;
-	// dK/dV kernel: order in which a key tile visits its (q-head, query tile) steps (see bwd_dkdv_tile), and whether a
-	// workgroup takes the key tiles p and ntiles - 1 - p one after the other (causal self-attention; a.mtiles then
-	// counts pairs)
-	int kv_order, kv_pair, kv_ntiles;  // kv_ntiles: key tiles per (batch, kv-head)
+	// dK/dV kernel: a workgroup takes the key tiles p and ntiles - 1 - p one after the other (causal self-attention;
+	// a.mtiles then counts pairs); kv_ntiles: key tiles per (batch, kv-head)
+	int kv_pair, kv_ntiles;
 	int fold_half;   // forward / dQ: workgroup ids from this one on are visited backwards (0 = off; see decode_block())
 	int interleave;  // xcd_remap 1: this many (batch, kv-head) groups of an XCD advance through their tiles together (1, 2 or 4)
 	int stages;      // backward: bit 0 delta, bit 1 dK/dV, bit 2 dQ
