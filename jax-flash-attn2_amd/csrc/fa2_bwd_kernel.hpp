@@ -142,6 +142,10 @@ FA2_DEV void bwd_dkdv_tile(const KArgs& a, const int nt, const int hk, const int
 	// dS = P * (dP accumulator).  The factor c1 = scale * log2(e) is applied to the fp32
 	// accumulator, as the reference scales the fp32 result of its dot (_backward_triton.py:554-559).
 	constexpr bool FOLD = KV_AGPR;
+	// Head dim 64 with bias, no dropout (matrix products through the compiler's builtins): the chain of dP still starts
+	// from -delta of the block's rows - the start value is the four LDS reads of the statistics as they are, the
+	// subtraction per value goes away (one of about eight vector-ALU instructions per value of a kernel that is bound by them).
+	constexpr bool FOLD_DEL = !FOLD && BIAS && !DROP && D == 64;
 	// Where the register files are left to the compiler it chooses accumulation registers for S / dP as well - results
 	// that the vector ALU consumes - and copies them out value by value; at head dim 256, where dK / dV fill the
 	// accumulation registers, it also moves 32 registers of dK / dV out of the way and back in every block (96 extra
@@ -296,7 +300,7 @@ FA2_DEV void bwd_dkdv_tile(const KArgs& a, const int nt, const int hk, const int
 	// lse in the units the elementwise stage wants, both negated where they start the chains
 	// (lse: -lse / (scale log2(e)) ... in the units of the raw dot product where it starts the chain of S, else -lse log2(e),
 	// the addend of the fused multiply-add that forms the exponent; delta: negated where it starts the chain of dP)
-	const float stat_mul = tid < BMQ ? (FOLD ? -inv_scale : -kLog2e) : (FOLD ? -1.f : 1.f);
+	const float stat_mul = tid < BMQ ? (FOLD ? -inv_scale : -kLog2e) : ((FOLD || FOLD_DEL) ? -1.f : 1.f);
 	auto store_stat = [&](float x, int buf) {
 		if (tid < 2 * BMQ) {
 			int which = tid / BMQ;
@@ -385,7 +389,12 @@ FA2_DEV void bwd_dkdv_tile(const KArgs& a, const int nt, const int hk, const int
 		// statistics of rows 8 aa + 4 g .. + 3 of block qb
 		auto issue_stat = [&](int qb, int aa) __attribute__((always_inline)) {
 			lse4[aa] = *(const FA2_LDS f32x4*)(stat + soff + (32 * qb + 8 * aa) * 4);
-			del4[aa] = *(const FA2_LDS f32x4*)(stat + soff + 2 * STAT_BYTES + (32 * qb + 8 * aa) * 4);
+			if constexpr (!FOLD_DEL) del4[aa] = *(const FA2_LDS f32x4*)(stat + soff + 2 * STAT_BYTES + (32 * qb + 8 * aa) * 4);
+		};
+		// FOLD_DEL: -delta of rows 8 aa + 4 g .. + 3 of block qb, the start value of its chain of dP (read a stage ahead of the statistics)
+		f32x4 cdel4[FOLD_DEL ? 4 : 1];
+		auto issue_del = [&](int qb, int aa) __attribute__((always_inline)) {
+			if constexpr (FOLD_DEL) cdel4[aa] = *(const FA2_LDS f32x4*)(stat + soff + 2 * STAT_BYTES + (32 * qb + 8 * aa) * 4);
 		};
 		// statistics of the quads whose phase 0 runs in slot j
 		auto issue_stat_for_slot = [&](int qb, int j) __attribute__((always_inline)) {
@@ -461,9 +470,12 @@ FA2_DEV void bwd_dkdv_tile(const KArgs& a, const int nt, const int hk, const int
 				f32x16 zero;
 #pragma unroll
 				for (int i = 0; i < 16; ++i) zero[i] = 0.f;
-				if (j & 1)
-					dpa = mfma32(afr[r], vf[ks], j == 1 ? zero : dpa);
-				else
+				if (j & 1) {
+					f32x16 c0 = zero;
+					if constexpr (FOLD_DEL)
+						c0 = __builtin_shufflevector(__builtin_shufflevector(cdel4[0], cdel4[1], 0, 1, 2, 3, 4, 5, 6, 7), __builtin_shufflevector(cdel4[2], cdel4[3], 0, 1, 2, 3, 4, 5, 6, 7), 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
+					dpa = mfma32(afr[r], vf[ks], j == 1 ? c0 : dpa);
+				} else
 					sa = mfma32(afr[r], kf[ks], j == 0 ? zero : sa);
 			}
 		};
@@ -581,7 +593,7 @@ FA2_DEV void bwd_dkdv_tile(const KArgs& a, const int nt, const int hk, const int
 				for (int e = e0; e < e1; ++e) {
 					// dP is read here, not in phase 0: the last product of its chain is then at
 					// least two matrix products back
-					if constexpr (!DROP) by[q][e] = dpa[4 * q + e] - del4[q][e];
+					if constexpr (!DROP) by[q][e] = FOLD_DEL ? dpa[4 * q + e] : dpa[4 * q + e] - del4[q][e];
 					float p = exp2_fast(bx[q][e]);
 					int row = m0 + 32 * qb + 8 * q + 4 * g + e;
 					if constexpr (MASKED) {
@@ -623,6 +635,10 @@ FA2_DEV void bwd_dkdv_tile(const KArgs& a, const int nt, const int hk, const int
 		if constexpr (FOLD) {
 #pragma unroll
 			for (int aa = 0; aa < 4; ++aa) issue_stat(0, aa);
+		}
+		if constexpr (FOLD_DEL) {
+#pragma unroll
+			for (int aa = 0; aa < 4; ++aa) issue_del(0, aa);
 		}
 
 		auto stage = [&](auto k_tag) __attribute__((always_inline)) {
@@ -669,6 +685,9 @@ FA2_DEV void bwd_dkdv_tile(const KArgs& a, const int nt, const int hk, const int
 					// the start values of the chains of the next block, in the last four slots
 					if constexpr (FOLD && NEXT_A) {
 						if (j >= NSLOT - 4) issue_stat(k + 1, j - (NSLOT - 4));
+					}
+					if constexpr (FOLD_DEL && NEXT_A) {
+						if (j >= NSLOT - 4) issue_del(k + 1, j - (NSLOT - 4));
 					}
 				}
 				// first half of the slot: product of A, first half of the micro-step(s) of B;
@@ -1160,7 +1179,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void bwd_dq_kernel(const KArgs a) {
 			for (int i = 0; i < 16; ++i) dq[qb][db][i] = 0.f;
 	// Without dropout the chain of dP starts from -delta of the lane's row (the 16 accumulator
 	// registers all belong to that row), so dS = P * (dP accumulator) without a subtraction.
-	constexpr bool FOLD_DP = !DROP && !BIAS && D <= 128;  // (the other variants have no registers to spare)
+	constexpr bool FOLD_DP = !DROP && D <= 128 && (!BIAS || D == 64);  // (head dim 128 with bias has no registers to spare: bound to 256, its variants spill as it is)
 	f32x16 ndel16[QB];
 #pragma unroll
 	for (int qb = 0; qb < QB; ++qb)
