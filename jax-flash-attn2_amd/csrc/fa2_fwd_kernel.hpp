@@ -738,7 +738,10 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 	// LDS read of a fragment PA products further on (a scheduling barrier after every slot pins that order).  The
 	// softmax is the path without the row maximum, applied per half; a half that needs the maximum after all (decided
 	// for the wave as a whole) takes it from its scores, which are still in their registers, before its P is used.
-	constexpr bool PIPE = D == 256 && NW == 4 && QB == 1 && FOLD && !SPLIT;
+	// (Head dim 128 takes the same path in its four-wave workgroups, where two waves share a SIMD: B4 H32 S4096 causal forward 0.531 -> 0.511 ms,
+	// B8 S2048 0.307 -> 0.294 ms; nothing at S 8192 or without a causal mask, and the eight-wave workgroups of long context
+	// measured 0.4 % slower and stay on the plain tile body.  With dropout the generator's pieces need sixteen slots a phase.)
+	constexpr bool PIPE = (D == 256 || (D == 128 && !DROP)) && NW == 4 && QB == 1 && FOLD && !SPLIT;
 	auto tile_pipe = [&](int n0) {
 		if constexpr (PIPE) {
 			constexpr int NFR = KS;  // fragments = products of a phase: KS of K for a half, 2 sixteen-key steps x DB of V
@@ -877,12 +880,28 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 			};
 			auto sv0 = [&](auto jt) __attribute__((always_inline)) {
 				constexpr int j = decltype(jt)::value;
-				if constexpr (j >= 2 && j < 10) soft_piece(0, j - 2);
+				if constexpr (NFR >= 10) {
+					if constexpr (j >= 2 && j < 10) soft_piece(0, j - 2);
+				} else {  // eight slots: the eight pieces behind the products 2 .. 7, two each behind the first two
+					if constexpr (j == 2 || j == 3) {
+						soft_piece(0, 2 * (j - 2));
+						soft_piece(0, 2 * (j - 2) + 1);
+					} else if constexpr (j >= 4)
+						soft_piece(0, j);
+				}
 				if constexpr (j >= 10) gen_piece(1, 0, std::integral_constant<int, j - 10>{});
 			};
 			auto sv1 = [&](auto jt) __attribute__((always_inline)) {
 				constexpr int j = decltype(jt)::value;
-				if constexpr (j >= 2 && j < 10) soft_piece(1, j - 2);
+				if constexpr (NFR >= 10) {
+					if constexpr (j >= 2 && j < 10) soft_piece(1, j - 2);
+				} else {
+					if constexpr (j == 2 || j == 3) {
+						soft_piece(1, 2 * (j - 2));
+						soft_piece(1, 2 * (j - 2) + 1);
+					} else if constexpr (j >= 4)
+						soft_piece(1, j);
+				}
 				if constexpr (j >= 10) gen_piece(1, 1, std::integral_constant<int, j - 10>{});
 			};
 #pragma unroll
