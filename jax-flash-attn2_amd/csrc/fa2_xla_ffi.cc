@@ -19,8 +19,8 @@
 //                 has_window bool, window_left i32, window_right i32, softcap f32
 // Every field of fa2_params is reachable: a `bias` buffer of element type PRED / U8 / S8 is a boolean mask, one
 // byte per position (bias_dtype = FA2_MASK_U8); `kv_lens` int32 [B]; the window and soft-capping are attributes;
-// `dbias` fp32 [B, Hq, Sq, Sk] is a result (0 elements = not wanted), cleared here by a fill kernel because the
-// dQ kernel leaves skipped key tiles unwritten.
+// `dbias`, fp32 in the shape of the bias, is a result (0 elements = not wanted), cleared here by a fill kernel because
+// the dQ kernel leaves skipped key tiles unwritten and adds into entries that several (batch, head) pairs share.
 // The dropout seed is an OPERAND (8 bytes on the device: u32[2] low word first, or one 64-bit
 // integer), as in the reference, whose custom call takes dropout_seed as an operand
 // (_forward_triton.py:553): a new seed then needs no new executable and the seed may be traced.
@@ -162,15 +162,17 @@ ffi::Error BwdImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::
 	p.scratch = scratch->untyped_data();
 	p.scratch_bytes = scratch->size_bytes();
 	if (dbias->element_count() > 0) {
-		// fp32 [B, Hq, Sq, Sk], dense; the dQ kernel leaves key tiles it skips unwritten: cleared first
+		// fp32, dense, in the shape of the bias ([B|1, Hq|Hkv|1, Sq, Sk]): stride 0 on its size-1 axes, where the dQ
+		// kernel accumulates over batch rows / heads itself; it leaves key tiles it skips unwritten: cleared first
 		auto dd = dbias->dimensions();
-		if (dd.size() != 4 || dbias->element_type() != ffi::DataType::F32 || dd[0] != p.B || dd[1] != p.Hq || dd[2] != p.Sq ||
-		    dd[3] != p.Sk || dd[3] % 4)
-			return ffi::Error(ffi::ErrorCode::kInvalidArgument, "dbias must be f32 [B, Hq, Sq, Sk] with Sk a multiple of 4");
+		auto bd = bias.dimensions();
+		if (dd.size() != 4 || bd.size() != 4 || dbias->element_type() != ffi::DataType::F32 || dd[0] != bd[0] || dd[1] != bd[1] ||
+		    dd[2] != p.Sq || dd[3] != p.Sk || dd[3] % 4)
+			return ffi::Error(ffi::ErrorCode::kInvalidArgument, "dbias must be f32 in the shape of the bias, Sk a multiple of 4");
 		p.dbias = (float*)dbias->untyped_data();
 		p.dbias_stride_m = dd[3];
-		p.dbias_stride_h = dd[2] * dd[3];
-		p.dbias_stride_b = dd[1] * dd[2] * dd[3];
+		p.dbias_stride_h = dd[1] == 1 ? 0 : dd[2] * dd[3];
+		p.dbias_stride_b = dd[0] == 1 ? 0 : dd[1] * dd[2] * dd[3];
 		size_t n16 = dbias->size_bytes() / 16;
 		size_t blocks = (n16 + 255) / 256;
 		hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)(blocks < 65535 ? blocks : 65535)), dim3(256), 0, stream, (uint4*)p.dbias, n16);

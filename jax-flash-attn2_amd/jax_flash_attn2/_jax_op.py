@@ -180,8 +180,9 @@ def _bwd_call(ops: dict, cfg: _Cfg):
 		dq=jax.ShapeDtypeStruct(q.shape, q.dtype),
 		dk=jax.ShapeDtypeStruct(k.shape, k.dtype),
 		dv=jax.ShapeDtypeStruct(v.shape, v.dtype),
-		# per-(batch, q-head) gradient of the additive term; 0 elements = not wanted
-		dbias=jax.ShapeDtypeStruct((B, Hq, Sq, Sk) if cfg.bias_grad else (0,), jnp.float32),
+		# gradient of the additive term, fp32, IN THE SHAPE OF THE BIAS (the kernels sum over the axes it is broadcast on);
+		# 0 elements = not wanted
+		dbias=jax.ShapeDtypeStruct(tuple(ops["bias"].shape) if cfg.bias_grad else (0,), jnp.float32),
 		scratch=jax.ShapeDtypeStruct((scratch_bytes,), jnp.uint8),
 	)
 	res = _ffi_call("fa2_bwd_ffi", tuple(out_types[n] for n in spec.BWD_RESULTS))(*[ops[n] for n in spec.BWD_OPERANDS], **_attr_dict(cfg))
@@ -203,27 +204,15 @@ def _attention_fwd(q, k, v, bias, seqlens, kv_lens, seed, cfg):
 
 def _attention_bwd(cfg, residual, dout):
 	q, k, v, bias, seqlens, kv_lens, seed, out, lse = residual
-	dq, dk, dv, dbias_full = _bwd_call(
+	dq, dk, dv, dbias32 = _bwd_call(
 		dict(q=q, k=k, v=v, bias=bias, seqlens=seqlens, kv_lens=kv_lens, seed=seed, o=out, lse=lse, dout=dout), cfg)
 	dbias = None  # the reference returns no gradient for the bias (_flash_attention.py:88); `bias_grad=True` asks for one
 	if cfg.bias_grad:
-		dbias = _reduce_dbias(dbias_full, bias.shape, k.shape[2]).astype(bias.dtype)
+		dbias = dbias32.astype(bias.dtype)
 	return dq, dk, dv, dbias, None, None, None
 
 
 _attention.defvjp(_attention_fwd, _attention_bwd)
-
-
-def _reduce_dbias(full, bias_shape, Hkv):
-	"""[B, Hq, Sq, Sk] per-head gradient -> the shape of the bias: summed over the axes the kernels broadcast it on."""
-	B, Hq = full.shape[:2]
-	if bias_shape[1] == 1:
-		full = full.sum(axis=1, keepdims=True)
-	elif bias_shape[1] != Hq:
-		full = full.reshape(B, Hkv, Hq // Hkv, *full.shape[2:]).sum(axis=2)
-	if bias_shape[0] == 1 and B != 1:
-		full = full.sum(axis=0, keepdims=True)
-	return full
 
 
 def flash_attention_call(q, k, v, attention_mask=None, bias=None, softmax_scale=None, dropout_prob=0.0, causal=False,

@@ -109,7 +109,7 @@ def test_forward_and_backward_calls_follow_the_binding_order(jop):
 	assert abs(float(attrs["softcap"]) - 30.0) < 1e-6 and abs(float(attrs["dropout_p"]) - 0.1) < 1e-6
 	res = dict(zip(spec.FWD_RESULTS, out_types))
 	assert res["o"].shape == q.shape and res["lse"].shape == (2, 4, 128) and res["scratch"].dtype == np.uint8
-	# the differentiation rule: same operands plus o, lse, dout; dbias as a result, reduced to the shape of the bias
+	# the differentiation rule: same operands plus o, lse, dout; dbias as a result in the shape of the bias
 	grads = mod._attention.pullback(np.ones_like(q))
 	name, operands, attrs, out_types, _ = calls[-1]
 	assert name == "fa2_bwd_ffi" and len(operands) == len(spec.BWD_OPERANDS)
@@ -117,7 +117,7 @@ def test_forward_and_backward_calls_follow_the_binding_order(jop):
 	assert ops["o"].shape == q.shape and ops["lse"].shape == (2, 4, 128) and ops["dout"].shape == q.shape
 	assert ops["seed"].tolist() == [7, 5] and ops["kv_lens"].tolist() == [100, 128]
 	res = dict(zip(spec.BWD_RESULTS, out_types))
-	assert res["dbias"].shape == (2, 4, 128, 128) and res["dbias"].dtype == np.float32
+	assert res["dbias"].shape == bias.shape and res["dbias"].dtype == np.float32  # not one entry per (batch, q-head)
 	assert res["dk"].shape == k.shape and res["dv"].shape == v.shape
 	dq, dk, dv, dbias, *rest = grads
 	assert dq.shape == q.shape and dk.shape == k.shape and dbias.shape == bias.shape and rest == [None, None, None]
