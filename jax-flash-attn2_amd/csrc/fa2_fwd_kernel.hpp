@@ -870,38 +870,34 @@ __global__ __launch_bounds__(NW * 64, WPS) void fwd_kernel(const KArgs a) {
 				});
 			};
 			auto none = [&](auto) __attribute__((always_inline)) {};
-			// the eight pieces of a half follow the products 2 .. 9 of the phase (the scores' last product is then at
-			// least two products back)
 			// (dropout: both calls of half 0 run in phase 0, the first call of half 1 at the end of phase 1, its second at the end of phase 2;
 			// the mask of a half is applied once its P is final: after soft_finish, before the phase that uses it)
 			auto gv0 = [&](auto jt) __attribute__((always_inline)) {
 				constexpr int j = decltype(jt)::value;
 				if constexpr (j < 12) gen_piece(0, j / 6, std::integral_constant<int, j % 6>{});
 			};
-			auto sv0 = [&](auto jt) __attribute__((always_inline)) {
+			// the eight softmax pieces of half hf behind the products of a phase (the scores' last product is then at least two
+			// products back): with sixteen slots one piece behind each of the products 2 .. 9, with eight slots (head dim 128)
+			// behind the products 2 .. 7, two each behind the first two (other distributions measured the same)
+			auto soft_slot = [&](int hf, auto jt) __attribute__((always_inline)) {
 				constexpr int j = decltype(jt)::value;
 				if constexpr (NFR >= 10) {
-					if constexpr (j >= 2 && j < 10) soft_piece(0, j - 2);
-				} else {  // eight slots: the eight pieces behind the products 2 .. 7, two each behind the first two
-					if constexpr (j == 2 || j == 3) {
-						soft_piece(0, 2 * (j - 2));
-						soft_piece(0, 2 * (j - 2) + 1);
-					} else if constexpr (j >= 4)
-						soft_piece(0, j);
+					if constexpr (j >= 2 && j < 10) soft_piece(hf, j - 2);
+				} else if constexpr (j == 2 || j == 3) {
+					soft_piece(hf, 2 * (j - 2));
+					soft_piece(hf, 2 * (j - 2) + 1);
+				} else if constexpr (j >= 4) {
+					soft_piece(hf, j);
 				}
+			};
+			auto sv0 = [&](auto jt) __attribute__((always_inline)) {
+				constexpr int j = decltype(jt)::value;
+				soft_slot(0, jt);
 				if constexpr (j >= 10) gen_piece(1, 0, std::integral_constant<int, j - 10>{});
 			};
 			auto sv1 = [&](auto jt) __attribute__((always_inline)) {
 				constexpr int j = decltype(jt)::value;
-				if constexpr (NFR >= 10) {
-					if constexpr (j >= 2 && j < 10) soft_piece(1, j - 2);
-				} else {
-					if constexpr (j == 2 || j == 3) {
-						soft_piece(1, 2 * (j - 2));
-						soft_piece(1, 2 * (j - 2) + 1);
-					} else if constexpr (j >= 4)
-						soft_piece(1, j);
-				}
+				soft_slot(1, jt);
 				if constexpr (j >= 10) gen_piece(1, 1, std::integral_constant<int, j - 10>{});
 			};
 #pragma unroll
