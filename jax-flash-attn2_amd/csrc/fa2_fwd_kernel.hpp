@@ -1141,13 +1141,17 @@ hipError_t launch_fwd_t(bool bias, bool drop, KArgs& a, hipStream_t s) {
 		// and V of a head stay in an XCD's L2 (4 MiB; B1 H4 S16384 D = 128, 8 MiB a head: 0.372 -> 0.568 ms).
 		// D = 64 keeps below 256 registers a wave in every variant and gains everywhere (B32 S512 H12 0.053 -> 0.045 ms,
 		// B128 S197 0.071 -> 0.056 ms, B4 S4096 Hq32 causal 0.377 -> 0.330 ms); D = 128 needs an instantiation bound to
-		// 256 registers, which the variants with bias do not fit, and gains under a causal mask (B8 S2048 0.330 -> 0.315 ms,
-		// B4 S4096 0.563 -> 0.552 ms) but not without at 2048 keys (0.536 -> 0.545 ms).
-		// (D = 128 at the limit, S = 8192: a grid of up to two such workgroups per CU still gains - B1 Hq8 0.193 -> 0.163 ms,
-		// the tail of 256 long workgroups is what costs there - a larger one does not, B2 Hq32 0.953 -> 0.971 ms)
-		const bool fits_l2 = (int64_t)a.Sk * D * 4 <= ((D == 128 && wgs > 2 * kNumCU) ? (2 << 20) : (4 << 20));
-		// (non-causal D = 128: up to 1024 keys, where the start and end of a workgroup weigh most - B16 S1024 0.316 -> 0.297 ms)
-		if (fits_l2 && (D == 64 || ((a.causal || a.Sk <= 1024) && !bias && !(a.softcap > 0.f))))
+		// 256 registers, which the variants with bias do not fit.  Its four-wave workgroups run their unmasked tiles
+		// through the pipelined path; with that they gain under a causal mask up to the 4 MiB (Hq32 Hkv8: B8 S2048 0.330 ->
+		// 0.303 ms, B4 S4096 0.563 -> 0.516 ms, B2 S8192 0.974 -> 0.965 ms, B2 S6144 Hq16 0.298 -> 0.280 ms; S16384 + 1 %) and
+		// without a mask up to 4096 keys (B8 S2048 0.520 -> 0.502 ms, B4 S4096 0.958 -> 0.953 ms; S8192 + 1 %).
+		// (With dropout the tiles keep the plain body and the limits measured for it: under a causal mask 2 MiB once the
+		// grid exceeds two workgroups per CU - B2 Hq32 S8192 0.953 -> 0.971 ms - and without a mask 1024 keys, where the
+		// start and end of a workgroup weigh most - B16 S1024 0.316 -> 0.297 ms.)
+		const int64_t kv_limit = D == 64   ? (4 << 20)
+		                         : a.causal ? ((drop && wgs > 2 * kNumCU) ? (2 << 20) : (4 << 20))
+		                                    : (drop ? 1024 * D * 4 : (2 << 20));
+		if ((int64_t)a.Sk * D * 4 <= kv_limit && (D == 64 || (!bias && !(a.softcap > 0.f))))
 			return launch_fwd_cfg<T, D, 4, (D == 128 ? 2 : 1)>(bias, drop, a, s);
 	}
 	return launch_fwd_cfg<T, D, C::NW, C::WPS>(bias, drop, a, s);
