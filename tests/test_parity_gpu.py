@@ -68,6 +68,9 @@ def test_large_logits(dtype, qk_scale, score_range):
 	# head dim 256, many tiles without masking: the row reference has to be raised in later tiles too (with and without dropout)
 	_run_case(1, 96, 448, 2, 1, 256, dtype, causal=False, qk_scale=qk_scale, p=0.1, seed=7, data_seed=4)
 	_run_case(1, 72, 520, 2, 2, 256, dtype, causal=False, qk_scale=qk_scale, data_seed=5)
+	# the same at head dim 128, whose four-wave workgroups take the pipelined path for tiles without masking
+	_run_case(1, 96, 448, 2, 1, 128, dtype, causal=False, qk_scale=qk_scale, data_seed=6)
+	_run_case(1, 200, 520, 4, 2, 128, dtype, causal=True, qk_scale=qk_scale, data_seed=7)
 
 
 @pytest.mark.parametrize(
